@@ -1,0 +1,119 @@
+/*
+ * libksana_sage_hip.so -- C ABI of the MI355X (gfx950) quantized "Sage" attention path.
+ *
+ * The reference (Tencent/KsanaDiT) has no FFI for this path: its Sage backend is a Python
+ * adaptor around one third-party call,
+ *     sageattn(q, k, v, tensor_layout="NHD", is_causal=...)
+ *         ksana/operations/attention/backends/sage_attn.py:75-81
+ * This library is what a Python backend class binds INSTEAD of that call.  The stage split
+ * (quantize Q/K, quantize V, fused attention) follows the stages visible at the reference's
+ * block-sparse sibling, ksana/operations/attention/backends/sage_sla.py:198-253.
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative KSANA_SAGE_E* code; it never throws,
+ *     exits or prints.  ksana_sage_last_error() gives the text for the calling thread.
+ *   - all work is enqueued on `stream` (a hipStream_t passed as void*) and the call returns
+ *     without synchronising.  The library allocates no device memory: the caller owns one
+ *     workspace blob whose size and sub-buffer offsets come from ksana_sage_workspace_layout().
+ *   - q, k, v, o are device pointers to [B, L, H, D] tensors of 16-bit floats (dtype below)
+ *     with strides given in ELEMENTS in that index order; the D stride must be 1, the
+ *     other strides multiples of 8 and the base pointers 16-byte aligned.
+ *   - inputs are never written.  Calls that share a workspace must be ordered on one stream.
+ */
+#ifndef KSANA_SAGE_HIP_H
+#define KSANA_SAGE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KSANA_SAGE_ABI_VERSION 1
+
+/* element types of q/k/v/o */
+#define KSANA_SAGE_BF16 0
+#define KSANA_SAGE_FP16 1
+
+/* error codes */
+#define KSANA_SAGE_OK 0
+#define KSANA_SAGE_EINVAL (-1)   /* bad shape, stride, alignment, dtype or null pointer      */
+#define KSANA_SAGE_ENOTSUP (-2)  /* valid request this build does not implement (D != 128, causal) */
+#define KSANA_SAGE_EHIP (-3)     /* the HIP runtime reported an error at launch               */
+
+/* rows per int8 scale: Q per token, K per 64 keys (sage_sla.py:190,204 uses (128, 64) off-Hopper;
+ * the per-token Q scale is free in this kernel's operand layout and tighter) */
+#define KSANA_SAGE_BLKQ 1
+#define KSANA_SAGE_BLKK 64
+
+typedef struct ksana_sage_shape {
+  int32_t B;   /* batch                                                     */
+  int32_t Hq;  /* query heads                                               */
+  int32_t Hkv; /* key/value heads; Hq % Hkv == 0                            */
+  int32_t Lq;  /* query sequence length                                     */
+  int32_t Lk;  /* key/value sequence length                                 */
+  int32_t D;   /* head size (128)                                           */
+} ksana_sage_shape;
+
+/* Byte offsets of the sub-buffers inside the workspace blob (each 256-byte aligned). */
+typedef struct ksana_sage_ws_layout {
+  uint64_t total_bytes;
+  uint64_t q_i8;    /* int8  [B, Hq, LqPad, D] row-major, LqPad = ceil(Lq/128)*128, pad rows 0 */
+  uint64_t q_scale; /* fp32  [B, Hq, LqPad]: one scale per query row                           */
+  uint64_t k_i8;    /* int8  [B, Hkv, nkb, 8192] nkb = ceil(Lk/64): one 64x128 tile per block,  */
+                    /*       stored in MFMA operand order (see ksanadit_amd/layout.py)          */
+  uint64_t k_scale; /* fp32  [B, Hkv, nkb]                                                      */
+  uint64_t k_mean;  /* fp32  [B, Hkv, D]: the channel mean AFTER rounding to the input dtype    */
+  uint64_t v_fp8;   /* e4m3fn[B, Hkv, nkb, 8192]: V^T tile 128x64 in MFMA operand order         */
+  uint64_t v_scale; /* fp32  [B, Hkv, D]                                                        */
+  uint64_t v_inv;   /* fp32  [B, Hkv, D]: 448/amax used by the V quantizer                      */
+  uint64_t k_part;  /* fp32  [B, Hkv, nch, D] nch = ceil(Lk/256): chunk sums of K               */
+  uint64_t v_part;  /* fp32  [B, Hkv, nch, D]: chunk abs-max of V                               */
+  int32_t lq_pad;
+  int32_t nqb;
+  int32_t nkb;
+  int32_t nch;
+} ksana_sage_ws_layout;
+
+/* Library identity.  No counterpart in the reference. */
+int ksana_sage_abi_version(void);
+const char* ksana_sage_last_error(void);
+
+/* Size/offsets of the scratch the stages below share.  Replaces the torch.empty calls the
+ * reference makes for its quantized operands (sage_sla.py:222-227). */
+int ksana_sage_workspace_layout(const ksana_sage_shape* shape, ksana_sage_ws_layout* out);
+
+/* Q -> Walsh-Hadamard transform over D, times sm_scale*log2(e)/128, per-row int8 + fp32 scale.
+ * Replaces the Q half of get_vanilla_qk_quant(q, k, km, 128, 64) (sage_sla.py:202-204). */
+int ksana_sage_quant_q(const void* q, int dtype, const int64_t q_strides[4], const ksana_sage_shape* shape,
+                       float sm_scale, void* workspace, void* stream);
+
+/* K -> channel mean over the sequence (km = k.mean(-2), sage_sla.py:198), subtracted when
+ * smooth_k != 0, then Walsh-Hadamard transform over D and per-64-row-block int8 + fp32 scale
+ * (K half of sage_sla.py:202-204). */
+int ksana_sage_quant_k(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
+                       int smooth_k, void* workspace, void* stream);
+
+/* V -> transposed, padded, operand-ordered fp8 e4m3fn with one fp32 scale per (b, h, d).
+ * Replaces transpose_pad_permute_cuda + scale_fuse_quant_cuda (sage_sla.py:222-228). */
+int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], const ksana_sage_shape* shape,
+                       void* workspace, void* stream);
+
+/* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
+ * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel
+ * call (sage_sla.py:237-253, dense form).  causal must be 0 in this build. */
+int ksana_sage_attn_fwd(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
+                        const ksana_sage_shape* shape, int causal, void* stream);
+
+/* The whole path in one call: quant_q, quant_k, quant_v, attn_fwd on `stream`.
+ * Replaces sageattn(q, k, v, tensor_layout="NHD", is_causal=causal) (sage_attn.py:75-81). */
+int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype,
+                       const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                       const int64_t o_strides[4], const ksana_sage_shape* shape, float sm_scale, int smooth_k,
+                       int causal, void* workspace, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KSANA_SAGE_HIP_H */

@@ -1,0 +1,114 @@
+"""ctypes binding of libksana_sage_hip.so (declared in include/ksana_sage_hip.h).
+
+The library is loaded once, from this package directory only (never from site-packages), and a
+missing or stale library is an error that names the build command - there is no CPU fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
+ABI_VERSION = 1
+
+BF16, FP16 = 0, 1
+OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
+
+EXPORTS = (
+    "ksana_sage_abi_version",
+    "ksana_sage_last_error",
+    "ksana_sage_workspace_layout",
+    "ksana_sage_quant_q",
+    "ksana_sage_quant_k",
+    "ksana_sage_quant_v",
+    "ksana_sage_attn_fwd",
+    "ksana_sage_forward",
+)
+
+
+class Shape(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("B", "Hq", "Hkv", "Lq", "Lk", "D")]
+
+
+class WsLayout(C.Structure):
+    _fields_ = [
+        (n, C.c_uint64)
+        for n in (
+            "total_bytes", "q_i8", "q_scale", "k_i8", "k_scale", "k_mean",
+            "v_fp8", "v_scale", "v_inv", "k_part", "v_part",
+        )
+    ] + [(n, C.c_int32) for n in ("lq_pad", "nqb", "nkb", "nch")]
+
+
+class SageLibraryError(RuntimeError):
+    """The HIP library is missing, stale, or rejected a call."""
+
+
+Strides = C.c_int64 * 4
+_lock = threading.Lock()
+_lib = None
+
+
+def _declare(lib):
+    vp, i, f = C.c_void_p, C.c_int, C.c_float
+    sp, lp, st = C.POINTER(Shape), C.POINTER(WsLayout), C.POINTER(C.c_int64)
+    lib.ksana_sage_abi_version.argtypes, lib.ksana_sage_abi_version.restype = [], i
+    lib.ksana_sage_last_error.argtypes, lib.ksana_sage_last_error.restype = [], C.c_char_p
+    lib.ksana_sage_workspace_layout.argtypes, lib.ksana_sage_workspace_layout.restype = [sp, lp], i
+    lib.ksana_sage_quant_q.argtypes, lib.ksana_sage_quant_q.restype = [vp, i, st, sp, f, vp, vp], i
+    lib.ksana_sage_quant_k.argtypes, lib.ksana_sage_quant_k.restype = [vp, i, st, sp, i, vp, vp], i
+    lib.ksana_sage_quant_v.argtypes, lib.ksana_sage_quant_v.restype = [vp, i, st, sp, vp, vp], i
+    lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, i, vp], i
+    lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, f, i, i, vp, vp]
+    lib.ksana_sage_forward.restype = i
+
+
+def library_present() -> bool:
+    return LIB_PATH.exists()
+
+
+def load():
+    """Return the loaded library; raise ``SageLibraryError`` when it cannot be used."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not LIB_PATH.exists():
+                raise SageLibraryError(
+                    f"{LIB_PATH} not found: build it with `python -m ksanadit_amd.build` (needs hipcc)"
+                )
+            try:
+                lib = C.CDLL(str(LIB_PATH))
+            except OSError as exc:
+                raise SageLibraryError(f"cannot load {LIB_PATH}: {exc}") from exc
+            missing = [n for n in EXPORTS if not hasattr(lib, n)]
+            if missing:
+                raise SageLibraryError(f"{LIB_PATH} lacks symbols {missing}: rebuild it")
+            _declare(lib)
+            if lib.ksana_sage_abi_version() != ABI_VERSION:
+                raise SageLibraryError(
+                    f"{LIB_PATH} has ABI {lib.ksana_sage_abi_version()}, this package needs {ABI_VERSION}: rebuild it"
+                )
+            _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    """Map a library return code to the exception the reference's callers expect."""
+    if rc == OK:
+        return
+    msg = f"{what}: {load().ksana_sage_last_error().decode()}"
+    if rc == EINVAL:
+        raise ValueError(msg)
+    if rc == ENOTSUP:
+        raise NotImplementedError(msg)
+    raise SageLibraryError(msg)
+
+
+def workspace_layout(B: int, Hq: int, Hkv: int, Lq: int, Lk: int, D: int) -> tuple[Shape, WsLayout]:
+    shape, layout = Shape(B, Hq, Hkv, Lq, Lk, D), WsLayout()
+    check(load().ksana_sage_workspace_layout(C.byref(shape), C.byref(layout)), "workspace_layout")
+    return shape, layout

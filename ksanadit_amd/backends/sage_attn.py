@@ -1,0 +1,69 @@
+"""Sage attention backend on the MI355X HIP library.
+
+Drop-in for ksana/operations/attention/backends/sage_attn.py:30-84: same class name, enum type,
+constructor and ``forward(query, key, value, **kwargs)``; tensors ``[B, L, H, D]``; inputs that
+are not fp16/bf16 are computed in bf16 and the result cast back (sage_attn.py:67-84); every
+backend kwarg the model blocks pass (``k_lens``, ``window_size``, ``latent_shape``, ``step_iter``,
+``block_id``, ``proj_l``, ``dense_only`` - ksana/models/wan/wan_model.py:182-189,240) is accepted
+and ignored, as the reference's adaptor ignores them.
+
+Differences, all deliberate:
+* the stored ``softmax_scale`` is USED (the reference stores it and lets the callee default to
+  ``D ** -0.5``; the two agree for every caller because attention_op.py:39 defaults to that value);
+* availability: no HIP device -> ``supports()`` is False and the selector moves on, like the
+  reference without its package (sage_attn.py:21-27,36-38); a HIP device with a missing or stale
+  library raises instead of falling back, so a broken build cannot hide behind another backend.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _capi, platform
+from ..config import KsanaAttentionBackend, KsanaAttentionConfig
+from ..sage_ops import sageattn
+from .base import KsanaAttentionBackendImpl
+
+SUPPORTED_HEAD_SIZES = (128,)
+
+
+class SageAttentionImpl(KsanaAttentionBackendImpl):
+    @staticmethod
+    def type() -> KsanaAttentionBackend:
+        return KsanaAttentionBackend.SAGE_ATTN
+
+    @staticmethod
+    def supports(**kwargs) -> bool:
+        if not platform.is_gpu():
+            return False
+        _capi.load()  # raises SageLibraryError on a GPU host whose library is missing or stale
+        head_size = kwargs.get("head_size")
+        return head_size is None or head_size in SUPPORTED_HEAD_SIZES
+
+    def __init__(
+        self,
+        attention_config: KsanaAttentionConfig,
+        num_heads: int,
+        head_size: int,
+        causal: bool,
+        softmax_scale: float,
+        num_kv_heads: int | None = None,
+        **extra_impl_args,
+    ) -> None:
+        if not platform.is_gpu():
+            raise RuntimeError("SageAttention backend requested but no HIP device is available.")
+        _capi.load()
+        if causal:
+            raise NotImplementedError("SageAttention HIP backend: causal masking is not implemented")
+        self.causal = causal
+        self.softmax_scale = softmax_scale
+        self.dropout = float(extra_impl_args.get("dropout_p", 0.0))
+        self.attention_config = attention_config
+        self.check_config()
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, **kwargs) -> torch.Tensor:
+        original_dtype = query.dtype
+        if original_dtype not in (torch.float16, torch.bfloat16):
+            query, key, value = (t.to(torch.bfloat16) for t in (query, key, value))
+        output = sageattn(query, key, value, tensor_layout="NHD", is_causal=self.causal, sm_scale=self.softmax_scale)
+        return output if output.dtype == original_dtype else output.to(original_dtype)

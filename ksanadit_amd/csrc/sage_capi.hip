@@ -1,0 +1,213 @@
+// C ABI of libksana_sage_hip.so: argument validation, workspace layout, kernel launches.
+// Declarations and the reference call sites each entry point replaces: include/ksana_sage_hip.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/ksana_sage_hip.h"
+#include "sage_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+uint64_t align256(uint64_t x) { return (x + 255u) & ~uint64_t(255); }
+
+int check_shape(const ksana_sage_shape* s) {
+  if (!s) return fail(KSANA_SAGE_EINVAL, "shape is null");
+  if (s->B < 1 || s->Hq < 1 || s->Hkv < 1 || s->Lq < 1 || s->Lk < 1)
+    return fail(KSANA_SAGE_EINVAL, "shape has a non-positive extent (B=%d Hq=%d Hkv=%d Lq=%d Lk=%d)", s->B, s->Hq,
+                s->Hkv, s->Lq, s->Lk);
+  if (s->Hq % s->Hkv != 0) return fail(KSANA_SAGE_EINVAL, "Hq=%d is not a multiple of Hkv=%d", s->Hq, s->Hkv);
+  if (s->D != ksana_sage::kD) return fail(KSANA_SAGE_ENOTSUP, "head size %d not supported (only 128)", s->D);
+  if ((int64_t)s->B * s->Hq > 65535 * 8 || s->Hq > 65535 || s->B > 65535)
+    return fail(KSANA_SAGE_EINVAL, "B*H too large for the launch grid");
+  return 0;
+}
+
+int check_tensor(const char* name, const void* ptr, int dtype, const int64_t st[4], int B, int L, int H) {
+  if (!ptr) return fail(KSANA_SAGE_EINVAL, "%s is null", name);
+  if (dtype != KSANA_SAGE_BF16 && dtype != KSANA_SAGE_FP16) return fail(KSANA_SAGE_EINVAL, "%s: dtype %d unknown", name, dtype);
+  if (!st) return fail(KSANA_SAGE_EINVAL, "%s: strides are null", name);
+  if (st[3] != 1) return fail(KSANA_SAGE_EINVAL, "%s: D stride is %lld, must be 1", name, (long long)st[3]);
+  if (reinterpret_cast<uintptr_t>(ptr) & 15u) return fail(KSANA_SAGE_EINVAL, "%s: pointer not 16-byte aligned", name);
+  const int ext[3] = {B, L, H};
+  for (int i = 0; i < 3; ++i) {
+    if (st[i] < 0) return fail(KSANA_SAGE_EINVAL, "%s: negative stride", name);
+    if (ext[i] > 1 && (st[i] % 8 != 0 || st[i] == 0))
+      return fail(KSANA_SAGE_EINVAL, "%s: stride[%d]=%lld must be a non-zero multiple of 8", name, i, (long long)st[i]);
+  }
+  return 0;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(KSANA_SAGE_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+ksana_sage::InTensor in_tensor(const void* p, int dtype, const int64_t st[4]) {
+  return ksana_sage::InTensor{static_cast<const uint16_t*>(p), st[0], st[1], st[2], dtype};
+}
+
+template <typename T>
+T* ws_at(void* ws, uint64_t off) {
+  return reinterpret_cast<T*>(static_cast<uint8_t*>(ws) + off);
+}
+template <typename T>
+const T* ws_at(const void* ws, uint64_t off) {
+  return reinterpret_cast<const T*>(static_cast<const uint8_t*>(ws) + off);
+}
+
+int check_ws(const void* ws) {
+  if (!ws) return fail(KSANA_SAGE_EINVAL, "workspace is null");
+  if (reinterpret_cast<uintptr_t>(ws) & 255u) return fail(KSANA_SAGE_EINVAL, "workspace not 256-byte aligned");
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ksana_sage_abi_version(void) { return KSANA_SAGE_ABI_VERSION; }
+
+const char* ksana_sage_last_error(void) { return g_err; }
+
+int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout* out) {
+  if (int rc = check_shape(s)) return rc;
+  if (!out) return fail(KSANA_SAGE_EINVAL, "layout out-pointer is null");
+  using namespace ksana_sage;
+  ksana_sage_ws_layout l;
+  memset(&l, 0, sizeof(l));
+  l.lq_pad = (s->Lq + kQPad - 1) / kQPad * kQPad;
+  l.nqb = l.lq_pad;  // one scale per (padded) query row
+  l.nkb = (s->Lk + kBlkK - 1) / kBlkK;
+  l.nch = (s->Lk + kMeanChunk - 1) / kMeanChunk;
+  const uint64_t bhq = (uint64_t)s->B * s->Hq, bhk = (uint64_t)s->B * s->Hkv;
+  uint64_t off = 0;
+  auto take = [&](uint64_t bytes) {
+    const uint64_t at = off;
+    off = align256(off + bytes);
+    return at;
+  };
+  l.q_i8 = take(bhq * l.lq_pad * kD);
+  l.q_scale = take(bhq * l.nqb * 4);
+  l.k_i8 = take(bhk * l.nkb * kTileBytes);
+  l.k_scale = take(bhk * l.nkb * 4);
+  l.k_mean = take(bhk * kD * 4);
+  l.v_fp8 = take(bhk * l.nkb * kTileBytes);
+  l.v_scale = take(bhk * kD * 4);
+  l.v_inv = take(bhk * kD * 4);
+  l.k_part = take(bhk * l.nch * kD * 4);
+  l.v_part = take(bhk * l.nch * kD * 4);
+  l.total_bytes = off;
+  *out = l;
+  return 0;
+}
+
+int ksana_sage_quant_q(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s, float sm_scale,
+                       void* ws, void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_tensor("q", q, dtype, st, s->B, s->Lq, s->Hq)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  ksana_sage_ws_layout l;
+  ksana_sage_workspace_layout(s, &l);
+  // one fp32 product, then an exact power of two (1/128 undoes the unnormalised Hadamard
+  // transforms of Q and K): part of the quantizer specification
+  const float premul = (sm_scale * 1.4426950408889634f) * 0.0078125f;
+  hipError_t e = ksana_sage::launch_quant_q(in_tensor(q, dtype, st), s->B, s->Hq, s->Lq, l.lq_pad, premul,
+                                            ws_at<int8_t>(ws, l.q_i8), ws_at<float>(ws, l.q_scale),
+                                            static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? 0 : hip_fail(e, "quant_q launch");
+}
+
+int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,
+                       void* ws, void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  ksana_sage_ws_layout l;
+  ksana_sage_workspace_layout(s, &l);
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  const ksana_sage::InTensor kt = in_tensor(k, dtype, st);
+  const int bhk = s->B * s->Hkv;
+  hipError_t e = hipSuccess;
+  if (smooth_k) {
+    e = ksana_sage::launch_col_partial(kt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.k_part), l.nch, hs);
+    if (e != hipSuccess) return hip_fail(e, "k column-sum launch");
+  }
+  e = ksana_sage::launch_k_mean_finalize(ws_at<float>(ws, l.k_part), bhk, smooth_k ? l.nch : 0, s->Lk, dtype,
+                                         smooth_k, ws_at<float>(ws, l.k_mean), hs);
+  if (e != hipSuccess) return hip_fail(e, "k mean finalize launch");
+  e = ksana_sage::launch_quant_k(kt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.k_mean),
+                                 ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs);
+  return e == hipSuccess ? 0 : hip_fail(e, "quant_k launch");
+}
+
+int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, void* ws,
+                       void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_tensor("v", v, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  ksana_sage_ws_layout l;
+  ksana_sage_workspace_layout(s, &l);
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  const ksana_sage::InTensor vt = in_tensor(v, dtype, st);
+  hipError_t e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, 1, ws_at<float>(ws, l.v_part), l.nch, hs);
+  if (e != hipSuccess) return hip_fail(e, "v abs-max launch");
+  e = ksana_sage::launch_v_scale_finalize(ws_at<float>(ws, l.v_part), s->B * s->Hkv, l.nch,
+                                          ws_at<float>(ws, l.v_scale), ws_at<float>(ws, l.v_inv), hs);
+  if (e != hipSuccess) return hip_fail(e, "v scale finalize launch");
+  e = ksana_sage::launch_quant_v(vt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.v_inv),
+                                 ws_at<uint8_t>(ws, l.v_fp8), hs);
+  return e == hipSuccess ? 0 : hip_fail(e, "quant_v launch");
+}
+
+int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
+                        int causal, void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
+  if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  ksana_sage_ws_layout l;
+  ksana_sage_workspace_layout(s, &l);
+  ksana_sage::AttnParams p;
+  p.q_i8 = ws_at<int8_t>(ws, l.q_i8);
+  p.q_scale = ws_at<float>(ws, l.q_scale);
+  p.k_tiles = ws_at<int8_t>(ws, l.k_i8);
+  p.k_scale = ws_at<float>(ws, l.k_scale);
+  p.v_tiles = ws_at<uint8_t>(ws, l.v_fp8);
+  p.v_scale = ws_at<float>(ws, l.v_scale);
+  p.o = ksana_sage::OutTensor{static_cast<uint16_t*>(o), o_st[0], o_st[1], o_st[2], dtype};
+  p.B = s->B, p.Hq = s->Hq, p.Hkv = s->Hkv, p.Lq = s->Lq, p.Lk = s->Lk;
+  p.lq_pad = l.lq_pad, p.nkb = l.nkb;
+  hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
+}
+
+int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
+                       const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
+                       const ksana_sage_shape* s, float sm_scale, int smooth_k, int causal, void* ws, void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
+  // validate everything before the first launch so a bad argument leaves no partial work
+  if (int rc = check_tensor("q", q, dtype, q_st, s->B, s->Lq, s->Hq)) return rc;
+  if (int rc = check_tensor("k", k, dtype, k_st, s->B, s->Lk, s->Hkv)) return rc;
+  if (int rc = check_tensor("v", v, dtype, v_st, s->B, s->Lk, s->Hkv)) return rc;
+  if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  if (int rc = ksana_sage_quant_q(q, dtype, q_st, s, sm_scale, ws, stream)) return rc;
+  if (int rc = ksana_sage_quant_k(k, dtype, k_st, s, smooth_k, ws, stream)) return rc;
+  if (int rc = ksana_sage_quant_v(v, dtype, v_st, s, ws, stream)) return rc;
+  return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, causal, stream);
+}
+
+}  // extern "C"

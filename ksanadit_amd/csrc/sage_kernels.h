@@ -1,0 +1,55 @@
+// Internal launch interface between the C ABI (sage_capi.hip) and the gfx950 kernels.
+// Pointers are device pointers; strides are in elements; every launcher enqueues on `stream`
+// and returns the hipError_t of the launch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ksana_sage {
+
+constexpr int kD = 128;          // head size the kernels are written for
+constexpr int kBlkQ = 1;         // query rows per int8 scale (per token)
+constexpr int kQPad = 128;       // stored query rows are padded to a multiple of this
+constexpr int kBlkK = 64;        // key rows per int8 scale == key rows per LDS tile
+constexpr int kMeanChunk = 256;  // rows per partial column sum
+constexpr int kTileBytes = kBlkK * kD;  // one K (int8) or V^T (fp8) tile: 8192 bytes
+constexpr int kAttnQPerWg = 256; // query rows per attention workgroup (8 waves x 32)
+
+struct InTensor {
+  const uint16_t* ptr;
+  int64_t sB, sL, sH;  // element strides of [B, L, H, D]; D stride is 1
+  int dtype;           // KSANA_SAGE_BF16 / KSANA_SAGE_FP16
+};
+
+struct OutTensor {
+  uint16_t* ptr;
+  int64_t sB, sL, sH;
+  int dtype;
+};
+
+// column reductions over the sequence: op 0 = ordered fp32 sum, op 1 = max of |x|
+hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s);
+hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
+                                  hipStream_t s);
+hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s);
+hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
+                          float* q_scale, hipStream_t s);
+hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
+                          float* k_scale, hipStream_t s);
+hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, uint8_t* v_tiles,
+                          hipStream_t s);
+
+struct AttnParams {
+  const int8_t* q_i8;
+  const float* q_scale;
+  const int8_t* k_tiles;
+  const float* k_scale;
+  const uint8_t* v_tiles;
+  const float* v_scale;
+  OutTensor o;
+  int B, Hq, Hkv, Lq, Lk, lq_pad, nkb;
+};
+hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s);
+
+}  // namespace ksana_sage

@@ -1,0 +1,385 @@
+// HBM-bound quantizer kernels for gfx950 (MI355X).
+//
+// Every kernel works on 128-channel rows of a [B, L, H, D] half tensor with the same thread
+// mapping: 256 threads = 32 row slots x 8 lanes, each lane owning 16 consecutive channels
+// (two 16-byte loads), so a wave reads four full 256-byte rows per load pair.
+//
+// The arithmetic is fixed to the last bit (it is compared bit-exactly with a PyTorch
+// specification): plain IEEE fp32 add / sub / mul / div, round-half-even, no contraction.
+#include "sage_kernels.h"
+
+#include "../../include/ksana_sage_hip.h"
+
+namespace ksana_sage {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kSlots = 32;  // row slots per workgroup
+
+template <int DT>
+__device__ __forceinline__ void widen8(const uint4& raw, float* out) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (DT == KSANA_SAGE_BF16) {
+      out[2 * i] = __uint_as_float(w[i] << 16);
+      out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    } else {
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      h2 p = __builtin_bit_cast(h2, w[i]);
+      out[2 * i] = (float)p[0];
+      out[2 * i + 1] = (float)p[1];
+    }
+  }
+}
+
+// 16 channels of one row; rows at or beyond L read as zero.
+template <int DT>
+__device__ __forceinline__ void load_row16(const uint16_t* row_ptr, bool valid, float* out) {
+  uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
+  if (valid) {
+    a = *reinterpret_cast<const uint4*>(row_ptr);
+    b = *reinterpret_cast<const uint4*>(row_ptr + 8);
+  }
+  widen8<DT>(a, out);
+  widen8<DT>(b, out + 8);
+}
+
+__device__ __forceinline__ float round_to_half_dtype(float x, int dtype) {
+  if (dtype == KSANA_SAGE_BF16) return (float)(__bf16)x;
+  return (float)(_Float16)x;
+}
+
+// ---------------------------------------------------------------------------------------
+// Column reduction over a chunk of 256 rows.  OP 0: fp32 sum in the frozen order (slot i%32
+// sequential over the chunk's 8 row groups, then an adjacent-pair tree over the 32 slots).
+// OP 1: max |x| (order free).  grid = (nch, H, B).
+// ---------------------------------------------------------------------------------------
+template <int DT, int OP>
+__global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
+                                                               int64_t sH, int H, int L, float* __restrict__ part,
+                                                               int nch) {
+  const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const uint16_t* base = x + b * sB + h * sH + c16 * 16;
+  float rows[kMeanChunk / kSlots][16];
+#pragma unroll
+  for (int i = 0; i < kMeanChunk / kSlots; ++i) {
+    const int row = ch * kMeanChunk + i * kSlots + slot;
+    load_row16<DT>(base + (int64_t)row * sL, row < L, rows[i]);
+  }
+  float acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = OP == 0 ? rows[0][e] : fabsf(rows[0][e]);
+#pragma unroll
+  for (int i = 1; i < kMeanChunk / kSlots; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = OP == 0 ? acc[e] + rows[i][e] : fmaxf(acc[e], fabsf(rows[i][e]));
+  }
+  // slots of one wave differ in lane bits 3..5
+#pragma unroll
+  for (int m = 8; m <= 32; m <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float o = __shfl_xor(acc[e], m);
+      acc[e] = OP == 0 ? acc[e] + o : fmaxf(acc[e], o);
+    }
+  }
+  __shared__ float s_w[4][kD];
+  const int wave = t >> 6, lane = t & 63;
+  if (lane < 8) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
+  }
+  __syncthreads();
+  if (t < kD) {
+    const float lo = OP == 0 ? s_w[0][t] + s_w[1][t] : fmaxf(s_w[0][t], s_w[1][t]);
+    const float hi = OP == 0 ? s_w[2][t] + s_w[3][t] : fmaxf(s_w[2][t], s_w[3][t]);
+    part[(((int64_t)b * H + h) * nch + ch) * kD + t] = OP == 0 ? lo + hi : fmaxf(lo, hi);
+  }
+}
+
+// chunk sums -> mean rounded to the input dtype, stored widened.  grid = B*H, 128 threads.
+__global__ __launch_bounds__(kD) void k_mean_finalize_kernel(const float* __restrict__ part, int nch, int L, int dtype,
+                                                             int smooth, float* __restrict__ k_mean) {
+  const int bh = blockIdx.x, d = threadIdx.x;
+  const float* p = part + (int64_t)bh * nch * kD + d;
+  float tot = nch > 0 ? p[0] : 0.0f;
+  for (int c = 1; c < nch; ++c) tot = tot + p[(int64_t)c * kD];
+  const float mean = __fdiv_rn(tot, (float)L);
+  k_mean[bh * kD + d] = smooth ? round_to_half_dtype(mean, dtype) : 0.0f;
+}
+
+__global__ __launch_bounds__(kD) void v_scale_finalize_kernel(const float* __restrict__ part, int nch,
+                                                              float* __restrict__ v_scale, float* __restrict__ v_inv) {
+  const int bh = blockIdx.x, d = threadIdx.x;
+  const float* p = part + (int64_t)bh * nch * kD + d;
+  float amax = p[0];
+  for (int c = 1; c < nch; ++c) amax = fmaxf(amax, p[(int64_t)c * kD]);
+  const bool nz = amax > 0.0f;
+  v_scale[bh * kD + d] = nz ? __fdiv_rn(amax, 448.0f) : 0.0f;
+  v_inv[bh * kD + d] = nz ? __fdiv_rn(448.0f, amax) : 0.0f;
+}
+
+// Unnormalised Walsh-Hadamard transform of one 128-channel row held by 8 adjacent lanes x 16
+// values (channel = 16*c16 + e).  Butterflies (a, b) -> (a + b, a - b) with stride 1, 2, 4, 8
+// inside the lane, then 16, 32, 64 across lanes c16 ^ 1, ^ 2, ^ 4 - in exactly that order.
+__device__ __forceinline__ void fwht128(float* x, int c16) {
+#pragma unroll
+  for (int s = 1; s < 16; s <<= 1) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if ((i & s) == 0) {
+        const float a = x[i], b = x[i + s];
+        x[i] = a + b;
+        x[i + s] = a - b;
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 1; m <= 4; m <<= 1) {
+    const bool upper = (c16 & m) != 0;  // this lane holds the "b" half of the pair
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float other = __shfl_xor(x[e], m);
+      const float own = upper ? -x[e] : x[e];
+      x[e] = other + own;
+    }
+  }
+}
+
+// max over the workgroup of a non-negative per-thread value
+__device__ __forceinline__ float block_max(float v, float* s_red) {
+#pragma unroll
+  for (int m = 1; m <= 32; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) s_red[wave] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+}
+
+__device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t acc = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float r = rintf(x[4 * i + j] * inv);
+      r = fminf(fmaxf(r, -127.0f), 127.0f);
+      acc |= ((uint32_t)(int)r & 0xffu) << (8 * j);
+    }
+    w[i] = acc;
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ---------------------------------------------------------------------------------------
+// Q: Hadamard transform, fold sm_scale*log2(e)/128, one int8 scale per query row.  One
+// workgroup handles 128 rows (4 per row slot).  grid = (lq_pad/128, H, B).  Output row-major
+// int8 [B, H, lq_pad, 128] and fp32 [B, H, lq_pad]; rows at or beyond L come out as zeros.
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __restrict__ q, int64_t sB, int64_t sL,
+                                                           int64_t sH, int H, int L, int lq_pad, float premul,
+                                                           int8_t* __restrict__ q_i8, float* __restrict__ q_scale) {
+  const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const uint16_t* base = q + b * sB + h * sH + c16 * 16;
+  constexpr int kRowsPerWg = 128, R = kRowsPerWg / kSlots;
+  const int64_t bh = (int64_t)b * H + h;
+  float x[R][16];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int row = blk * kRowsPerWg + i * kSlots + slot;
+    load_row16<DT>(base + (int64_t)row * sL, row < L, x[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int row = blk * kRowsPerWg + i * kSlots + slot;
+    fwht128(x[i], c16);
+    float amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      x[i][e] = x[i][e] * premul;
+      amax = fmaxf(amax, fabsf(x[i][e]));
+    }
+#pragma unroll
+    for (int m = 1; m <= 4; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
+    const bool nz = amax > 0.0f;
+    const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
+    if (c16 == 0) q_scale[bh * lq_pad + row] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
+    *reinterpret_cast<uint4*>(q_i8 + (bh * lq_pad + row) * kD + c16 * 16) = pack_int8x16(x[i], inv);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// K: subtract the channel mean, Hadamard transform, one int8 scale per 64-row block = one
+// workgroup.  grid = (nkb, H, B).  The tile is written in the order
+// the attention kernel's int8 MFMA consumes it: fragment (t = row/32, s = 32-channel step)
+// is 64 lanes x 16 bytes, lane = 32*(16-channel half within the step) + row%32.
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
+                                                           int64_t sH, int H, int L, int nkb,
+                                                           const float* __restrict__ k_mean,
+                                                           int8_t* __restrict__ k_tiles, float* __restrict__ k_scale) {
+  const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int64_t bh = (int64_t)b * H + h;
+  const uint16_t* base = k + b * sB + h * sH + c16 * 16;
+  float km[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) km[e] = k_mean[bh * kD + c16 * 16 + e];
+  constexpr int R = kBlkK / kSlots;
+  float x[R][16];
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int row = blk * kBlkK + i * kSlots + slot;
+    const bool valid = row < L;
+    load_row16<DT>(base + (int64_t)row * sL, valid, x[i]);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      x[i][e] = valid ? x[i][e] - km[e] : 0.0f;
+    }
+    fwht128(x[i], c16);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(x[i][e]));
+  }
+  __shared__ float s_red[4];
+  amax = block_max(amax, s_red);
+  const bool nz = amax > 0.0f;
+  const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
+  if (t == 0) k_scale[bh * nkb + blk] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
+  int8_t* tile = k_tiles + (bh * nkb + blk) * (int64_t)kTileBytes;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int frag = i * 4 + (c16 >> 1);
+    const int lane = (c16 & 1) * 32 + slot;
+    *reinterpret_cast<uint4*>(tile + (frag * 64 + lane) * 16) = pack_int8x16(x[i], inv);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// V: one workgroup per 64-row block.  grid = (nkb, H, B).  Scales with 448/amax[d], converts
+// to e4m3fn, transposes through LDS and writes the V^T tile in the order the fp8 MFMA
+// consumes it: chunk (dt = d/32, tt = half of the 64 rows) is 64 lanes x 16 bytes,
+// lane = 32*hh + d%32, byte r <-> row 32*tt + 8*(r/4) + 4*hh + r%4.
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __restrict__ v, int64_t sB, int64_t sL,
+                                                           int64_t sH, int H, int L, int nkb,
+                                                           const float* __restrict__ v_inv,
+                                                           uint8_t* __restrict__ v_tiles) {
+  const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int64_t bh = (int64_t)b * H + h;
+  const uint16_t* base = v + b * sB + h * sH + c16 * 16;
+  constexpr int kStride = kD + 16;  // LDS row pitch in bytes
+  __shared__ __attribute__((aligned(16))) uint8_t s_v[kBlkK * kStride];
+  float inv[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) inv[e] = v_inv[bh * kD + c16 * 16 + e];
+#pragma unroll
+  for (int i = 0; i < kBlkK / kSlots; ++i) {
+    const int r = i * kSlots + slot;
+    const int row = blk * kBlkK + r;
+    float x[16];
+    load_row16<DT>(base + (int64_t)row * sL, row < L, x);
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float y[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = fminf(fmaxf(x[4 * j + e] * inv[4 * j + e], -448.0f), 448.0f);
+      int packed = 0;
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], packed, false);
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], packed, true);
+      w[j] = (uint32_t)packed;
+    }
+    *reinterpret_cast<uint4*>(&s_v[r * kStride + c16 * 16]) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  __syncthreads();
+  uint8_t* tile = v_tiles + (bh * nkb + blk) * (int64_t)kTileBytes;
+#pragma unroll
+  for (int i = 0; i < kTileBytes / 16 / kThreads; ++i) {
+    const int oc = i * kThreads + t;
+    const int dt = oc >> 7, tt = (oc >> 6) & 1, lane = oc & 63;
+    const int hh = lane >> 5, d = dt * 32 + (lane & 31);
+    uint32_t w[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint32_t acc = 0;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int row = 32 * tt + 8 * g + 4 * hh + c;
+        acc |= (uint32_t)s_v[row * kStride + d] << (8 * c);
+      }
+      w[g] = acc;
+    }
+    *reinterpret_cast<uint4*>(tile + oc * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+}  // namespace
+
+#define KSANA_DISPATCH_DT(dtype, ...)            \
+  do {                                           \
+    if ((dtype) == KSANA_SAGE_BF16) {            \
+      constexpr int DT = KSANA_SAGE_BF16;        \
+      __VA_ARGS__;                               \
+    } else {                                     \
+      constexpr int DT = KSANA_SAGE_FP16;        \
+      __VA_ARGS__;                               \
+    }                                            \
+  } while (0)
+
+hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s) {
+  const dim3 grid(nch, H, B), block(kThreads);
+  KSANA_DISPATCH_DT(x.dtype, {
+    if (op == 0)
+      col_partial_kernel<DT, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch);
+    else
+      col_partial_kernel<DT, 1><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch);
+  });
+  return hipGetLastError();
+}
+
+hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
+                                  hipStream_t s) {
+  k_mean_finalize_kernel<<<dim3(BH), dim3(kD), 0, s>>>(part, nch, L, dtype, smooth, k_mean);
+  return hipGetLastError();
+}
+
+hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s) {
+  v_scale_finalize_kernel<<<dim3(BH), dim3(kD), 0, s>>>(part, nch, v_scale, v_inv);
+  return hipGetLastError();
+}
+
+hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
+                          float* q_scale, hipStream_t s) {
+  const dim3 grid(lq_pad / 128, H, B), block(kThreads);
+  KSANA_DISPATCH_DT(q.dtype,
+                    (quant_q_kernel<DT><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8,
+                                                               q_scale)));
+  return hipGetLastError();
+}
+
+hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
+                          float* k_scale, hipStream_t s) {
+  const dim3 grid(nkb, H, B), block(kThreads);
+  KSANA_DISPATCH_DT(k.dtype, (quant_k_kernel<DT><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean,
+                                                                         k_tiles, k_scale)));
+  return hipGetLastError();
+}
+
+hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, uint8_t* v_tiles,
+                          hipStream_t s) {
+  const dim3 grid(nkb, H, B), block(kThreads);
+  KSANA_DISPATCH_DT(v.dtype,
+                    (quant_v_kernel<DT><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, v_inv, v_tiles)));
+  return hipGetLastError();
+}
+
+}  // namespace ksana_sage

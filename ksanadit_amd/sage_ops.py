@@ -1,0 +1,189 @@
+"""Python face of the HIP library: the functions a backend (or a test) calls.
+
+``sageattn`` has the signature of the third-party function the reference's backend calls
+(``sageattn(q, k, v, tensor_layout="NHD", is_causal=...)``,
+ksana/operations/attention/backends/sage_attn.py:75-81); the stage functions expose the quantized
+operands so they can be compared bit for bit with a specification.
+
+Everything runs on the tensors' HIP device, on torch's current stream, without synchronising.
+Scratch comes from torch's caching allocator, so it is stream-ordered and recycled across the
+thousands of calls of one generation.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+
+from . import _capi
+from .layout import TILE_BYTES
+
+_DTYPES = {torch.bfloat16: _capi.BF16, torch.float16: _capi.FP16}
+
+
+def _strides(t: torch.Tensor):
+    return _capi.Strides(*t.stride())
+
+
+def _usable(t: torch.Tensor) -> torch.Tensor:
+    """The kernels read 16 bytes at a time along D: fix up layouts that do not allow it."""
+    s = t.stride()
+    ok = s[3] == 1 and all(x % 8 == 0 and x > 0 for x, n in zip(s[:3], t.shape[:3]) if n > 1)
+    if ok and t.data_ptr() % 16 == 0:
+        return t
+    return t.contiguous()
+
+
+def _stream_ptr(device) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_hip(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(
+                "the Sage HIP backend needs tensors on a HIP device; there is no CPU path "
+                f"(got device {t.device})"
+            )
+    if len({t.device for t in tensors}) != 1 or len({t.dtype for t in tensors}) != 1:
+        raise ValueError("q, k, v must share one device and one dtype")
+    if tensors[0].dtype not in _DTYPES:
+        raise ValueError(f"dtype {tensors[0].dtype} not supported by the kernels (bf16 / fp16 only)")
+
+
+@dataclass
+class SageWorkspace:
+    """One scratch blob plus typed views of its sub-buffers (see include/ksana_sage_hip.h)."""
+
+    shape: _capi.Shape
+    layout: _capi.WsLayout
+    blob: torch.Tensor
+
+    @classmethod
+    def allocate(cls, B, Hq, Hkv, Lq, Lk, D, device) -> "SageWorkspace":
+        shape, layout = _capi.workspace_layout(B, Hq, Hkv, Lq, Lk, D)
+        blob = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+        if blob.data_ptr() % 256:
+            raise RuntimeError("allocator returned a workspace that is not 256-byte aligned")
+        return cls(shape, layout, blob)
+
+    @property
+    def ptr(self) -> C.c_void_p:
+        return C.c_void_p(self.blob.data_ptr())
+
+    def _view(self, off: int, nbytes: int, dtype, shape):
+        return self.blob[off : off + nbytes].view(dtype).view(shape)
+
+    @property
+    def q_i8(self):
+        s, l = self.shape, self.layout
+        return self._view(l.q_i8, s.B * s.Hq * l.lq_pad * s.D, torch.int8, (s.B, s.Hq, l.lq_pad, s.D))
+
+    @property
+    def q_scale(self):
+        s, l = self.shape, self.layout
+        return self._view(l.q_scale, s.B * s.Hq * l.lq_pad * 4, torch.float32, (s.B, s.Hq, l.lq_pad))
+
+    @property
+    def k_tiles(self):
+        s, l = self.shape, self.layout
+        return self._view(l.k_i8, s.B * s.Hkv * l.nkb * TILE_BYTES, torch.int8, (s.B, s.Hkv, l.nkb, TILE_BYTES))
+
+    @property
+    def k_scale(self):
+        s, l = self.shape, self.layout
+        return self._view(l.k_scale, s.B * s.Hkv * l.nkb * 4, torch.float32, (s.B, s.Hkv, l.nkb))
+
+    @property
+    def k_mean(self):
+        s, l = self.shape, self.layout
+        return self._view(l.k_mean, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
+
+    @property
+    def v_tiles(self):
+        s, l = self.shape, self.layout
+        return self._view(l.v_fp8, s.B * s.Hkv * l.nkb * TILE_BYTES, torch.uint8, (s.B, s.Hkv, l.nkb, TILE_BYTES))
+
+    @property
+    def v_scale(self):
+        s, l = self.shape, self.layout
+        return self._view(l.v_scale, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
+
+
+def workspace_for(q: torch.Tensor, k: torch.Tensor) -> SageWorkspace:
+    B, Lq, Hq, D = q.shape
+    _, Lk, Hkv, _ = k.shape
+    return SageWorkspace.allocate(B, Hq, Hkv, Lq, Lk, D, q.device)
+
+
+def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float) -> None:
+    _require_hip(q)
+    q = _usable(q)
+    lib = _capi.load()
+    rc = lib.ksana_sage_quant_q(q.data_ptr(), _DTYPES[q.dtype], _strides(q), C.byref(ws.shape), sm_scale, ws.ptr,
+                                _stream_ptr(q.device))
+    _capi.check(rc, "ksana_sage_quant_q")
+
+
+def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True) -> None:
+    _require_hip(k)
+    k = _usable(k)
+    lib = _capi.load()
+    rc = lib.ksana_sage_quant_k(k.data_ptr(), _DTYPES[k.dtype], _strides(k), C.byref(ws.shape), int(smooth_k), ws.ptr,
+                                _stream_ptr(k.device))
+    _capi.check(rc, "ksana_sage_quant_k")
+
+
+def quant_v(v: torch.Tensor, ws: SageWorkspace) -> None:
+    _require_hip(v)
+    v = _usable(v)
+    lib = _capi.load()
+    rc = lib.ksana_sage_quant_v(v.data_ptr(), _DTYPES[v.dtype], _strides(v), C.byref(ws.shape), ws.ptr,
+                                _stream_ptr(v.device))
+    _capi.check(rc, "ksana_sage_quant_v")
+
+
+def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False) -> torch.Tensor:
+    _require_hip(out)
+    lib = _capi.load()
+    rc = lib.ksana_sage_attn_fwd(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
+                                 int(causal), _stream_ptr(out.device))
+    _capi.check(rc, "ksana_sage_attn_fwd")
+    return out
+
+
+def sageattn(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    tensor_layout: str = "NHD",
+    is_causal: bool = False,
+    sm_scale: float | None = None,
+    smooth_k: bool = True,
+    workspace: SageWorkspace | None = None,
+) -> torch.Tensor:
+    """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out."""
+    if tensor_layout not in ("NHD", "HND"):
+        raise ValueError(f"tensor_layout {tensor_layout!r} unknown")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("sageattn expects 4-D tensors")
+    if tensor_layout == "HND":
+        q, k, v = (t.transpose(1, 2) for t in (q, k, v))
+    _require_hip(q, k, v)
+    if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
+        raise ValueError(f"incompatible shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+    q, k, v = _usable(q), _usable(k), _usable(v)
+    B, Lq, Hq, D = q.shape
+    sm_scale = D**-0.5 if sm_scale is None else float(sm_scale)
+    ws = workspace_for(q, k) if workspace is None else workspace
+    out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
+    lib = _capi.load()
+    rc = lib.ksana_sage_forward(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
+        _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape),
+        sm_scale, int(smooth_k), int(is_causal), ws.ptr, _stream_ptr(q.device),
+    )
+    _capi.check(rc, "ksana_sage_forward")
+    return out.transpose(1, 2) if tensor_layout == "HND" else out

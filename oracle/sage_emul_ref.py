@@ -1,0 +1,62 @@
+"""Oracle: dequantised emulation of the fused Sage attention kernel.  Test infrastructure only.
+
+Stage (a6.4) of the path: what the third-party kernel called at
+ksana/operations/attention/backends/sage_attn.py:75-81 computes, with the operand roles of
+the kernel signature visible at sage_sla.py:237-253 (q_int8, k_int8, v_fp8, q_scale, k_scale,
+v_scale):
+
+    S  = (Q_i8 . K_i8^T) * q_scale * k_scale        integer dot products, exact
+    P  = exp2(S - rowmax(S) + P_SHIFT)              Q already carries sm_scale * log2(e)
+    O  = (fp8(P) . V_fp8) * v_scale / rowsum(P)
+
+It uses a full (not online) softmax in fp32, so it separates "error of the quantised
+scheme" from "bug in the kernel": the HIP kernel must agree with this far more tightly than
+either agrees with SDPA.  It is an approximation of SDPA by construction and is pinned by
+its distance to ``sdpa_ref`` plus exact invariants (see tests/test_oracle.py).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .quant_ref import BLKK, BLKQ, FP8_MAX, quant_k_ref, quant_q_ref, quant_v_ref
+
+# P is scaled by 2**P_SHIFT before the fp8 cast so that small probabilities stay above the
+# e4m3 subnormal floor (2**-9); the factor cancels in O = (P V) / rowsum(P).
+P_SHIFT = 8.0
+
+
+def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False):
+    """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``."""
+    B, H, Lq, D = q_i8.shape
+    Hkv, Lk = k_i8.shape[1], k_i8.shape[2]
+    g = H // Hkv
+    out = torch.empty(B, Lq, H, D, dtype=out_dtype)
+    qs_row = q_scale.repeat_interleave(BLKQ, dim=2)[:, :, :Lq]  # [B, H, Lq] (BLKQ == 1: already per row)
+    ks_col = k_scale.repeat_interleave(BLKK, dim=2)[:, :, :Lk]  # [B, Hkv, Lk]
+    for b in range(B):
+        for h in range(H):
+            hk = h // g
+            # int8 x int8 sums stay below 2**24, so fp32 matmul is exact here
+            s_int = q_i8[b, h].float() @ k_i8[b, hk].float().t()
+            s = s_int * (qs_row[b, h][:, None] * ks_col[b, hk][None, :])
+            if causal:
+                mask = torch.ones(Lq, Lk, dtype=torch.bool).tril(diagonal=Lk - Lq)
+                s = s.masked_fill(~mask, float("-inf"))
+            m = s.amax(dim=1, keepdim=True)
+            p = torch.exp2(s - m + P_SHIFT)
+            l = p.sum(dim=1, keepdim=True)
+            p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+            o = (p8 @ v_fp8[b, hk].float()) * v_scale[b, hk][None, :] / l
+            out[b, :, h, :] = o.to(out_dtype)
+    return out
+
+
+def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False):
+    """[B, L, H, D] half in, same out: quantise with the oracle quantizer, then emulate."""
+    D = q.shape[-1]
+    sm_scale = D**-0.5 if sm_scale is None else sm_scale
+    q_i8, q_scale = quant_q_ref(q, sm_scale)
+    k_i8, k_scale, _ = quant_k_ref(k, smooth_k=smooth_k)
+    v_fp8, v_scale = quant_v_ref(v)
+    return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal)

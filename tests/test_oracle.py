@@ -1,0 +1,352 @@
+"""Pins the CPU oracle itself (no GPU): every oracle function is checked against something that
+is NOT a retyping of its own formula - a float64 brute force, a scalar pure-Python second
+implementation that replays the specified order element by element, hand-computed blocks, the
+fp8 format definition, and invariants the mathematics fixes."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant_ref as qr
+from oracle.sage_emul_ref import sage_emul_ref
+from oracle.sdpa_ref import attention_bruteforce_f64, sdpa_ref, sdpa_ref_fp32
+
+f32 = np.float32
+
+
+def _rand(shape, seed, dtype=torch.bfloat16, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std).to(dtype)
+
+
+# ------------------------------------------------------------------ sdpa_ref
+@pytest.mark.parametrize("B,Lq,Lk,H,Hkv,D", [(1, 17, 17, 2, 2, 16), (2, 33, 20, 4, 2, 32), (1, 8, 50, 3, 3, 128)])
+def test_sdpa_ref_matches_f64_bruteforce(B, Lq, Lk, H, Hkv, D):
+    q, k, v = _rand((B, Lq, H, D), 1, torch.float32), _rand((B, Lk, Hkv, D), 2, torch.float32), _rand((B, Lk, Hkv, D), 3, torch.float32)
+    ref = attention_bruteforce_f64(q, k, v)
+    out = sdpa_ref(q, k, v)
+    assert out.shape == q.shape
+    torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=1e-5)
+    out_scaled = sdpa_ref(q, k, v, scale=0.3)
+    torch.testing.assert_close(out_scaled.double(), attention_bruteforce_f64(q, k, v, scale=0.3), rtol=1e-5, atol=1e-5)
+
+
+def test_sdpa_ref_causal_and_half():
+    q, k, v = (_rand((1, 24, 2, 32), s, torch.float32) for s in (4, 5, 6))
+    torch.testing.assert_close(sdpa_ref(q, k, v, causal=True).double(), attention_bruteforce_f64(q, k, v, causal=True), rtol=1e-5, atol=1e-5)
+    qb, kb, vb = (t.to(torch.bfloat16) for t in (q, k, v))
+    out = sdpa_ref(qb, kb, vb)
+    assert out.dtype == torch.bfloat16
+    assert (out.double() - attention_bruteforce_f64(qb, kb, vb)).abs().max() < 2e-2
+    torch.testing.assert_close(sdpa_ref_fp32(qb, kb, vb).double(), attention_bruteforce_f64(qb, kb, vb), rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------ K mean
+def _scalar_mean_sum(col):
+    """Replay rule 1 for ONE column with numpy float32 scalars."""
+    L = len(col)
+    nch = (L + qr.MEAN_CHUNK - 1) // qr.MEAN_CHUNK
+    tot = None
+    for c in range(nch):
+        slots = []
+        for s in range(qr.MEAN_SLOTS):
+            acc = None
+            for i in range(qr.MEAN_CHUNK // qr.MEAN_SLOTS):
+                r = c * qr.MEAN_CHUNK + i * qr.MEAN_SLOTS + s
+                x = f32(col[r]) if r < L else f32(0.0)
+                acc = x if acc is None else f32(acc + x)
+            slots.append(acc)
+        while len(slots) > 1:
+            slots = [f32(slots[i] + slots[i + 1]) for i in range(0, len(slots), 2)]
+        tot = slots[0] if tot is None else f32(tot + slots[0])
+    return tot
+
+
+@pytest.mark.parametrize("L", [1, 31, 256, 257, 700])
+def test_k_mean_matches_scalar_replay(L):
+    k = _rand((1, L, 2, 4), 10 + L, std=3.0) + 5.0
+    tot = qr.k_mean_sum_ref(k)
+    km = qr.k_mean_ref(k)
+    for h in range(2):
+        for d in range(4):
+            col = k[0, :, h, d].float().numpy()
+            s = _scalar_mean_sum(col)
+            assert tot[0, h, d].item() == float(s), (h, d)
+            mean = f32(s / f32(L))
+            expect = torch.tensor(float(mean)).to(torch.bfloat16)
+            assert km[0, h, d].item() == expect.item()
+
+
+def test_k_mean_close_to_f64_and_constant_columns():
+    k = _rand((2, 5000, 3, 8), 77, std=2.0) + 3.0
+    km = qr.k_mean_ref(k).double()
+    exact = k.double().mean(dim=1)
+    assert (km - exact).abs().max() <= exact.abs().max() * 2**-8  # one bf16 rounding
+    tot = qr.k_mean_sum_ref(k).double()
+    assert ((tot - k.double().sum(dim=1)).abs() / k.double().abs().sum(dim=1)).max() < 1e-6
+    const = torch.full((1, 777, 1, 4), 1.5, dtype=torch.bfloat16)
+    assert torch.equal(qr.k_mean_ref(const), torch.full((1, 1, 4), 1.5, dtype=torch.bfloat16))
+    assert qr.k_mean_ref(k.to(torch.float16)).dtype == torch.float16
+
+
+# ------------------------------------------------------------------ int8 block quantizer
+def _scalar_block_int8(x2d, blk):
+    """Independent scalar implementation of rule 4 on a [L, D] float32 numpy array."""
+    L, D = x2d.shape
+    nb = (L + blk - 1) // blk
+    out = np.zeros((L, D), dtype=np.int8)
+    scales = np.zeros(nb, dtype=np.float32)
+    for b in range(nb):
+        rows = range(b * blk, min(L, (b + 1) * blk))
+        amax = f32(0.0)
+        for r in rows:
+            for d in range(D):
+                a = f32(abs(x2d[r, d]))
+                if a > amax:
+                    amax = a
+        if amax == 0:
+            continue
+        scales[b] = f32(amax / f32(127.0))
+        inv = f32(f32(127.0) / amax)
+        for r in rows:
+            for d in range(D):
+                y = f32(x2d[r, d] * inv)
+                n = float(np.rint(y))  # rint = half to even
+                out[r, d] = int(max(-127.0, min(127.0, n)))
+    return out, scales
+
+
+# ------------------------------------------------------------------ Walsh-Hadamard stage
+def _sylvester(n):
+    return np.array([[(-1) ** bin(i & j).count("1") for j in range(n)] for i in range(n)], dtype=np.float64)
+
+
+def _scalar_fwht(row):
+    """Replay rule 3 on one row with float32 scalars: strides 1, 2, 4, ... in that order."""
+    x = [f32(v) for v in row]
+    n, s = len(x), 1
+    while s < n:
+        for base in range(0, n, 2 * s):
+            for i in range(base, base + s):
+                a, b = x[i], x[i + s]
+                x[i], x[i + s] = f32(a + b), f32(a - b)
+        s *= 2
+    return np.array(x, dtype=np.float32)
+
+
+def test_fwht_is_the_hadamard_matrix_in_natural_order():
+    g = torch.Generator().manual_seed(8)
+    xi = torch.randint(-50, 50, (5, 128), generator=g).float()  # integers: every butterfly is exact
+    assert np.array_equal(qr.fwht_ref(xi).double().numpy(), xi.double().numpy() @ _sylvester(128))
+    x = _rand((3, 7, 128), 12, torch.float32, std=3.0)
+    y = qr.fwht_ref(x)
+    np.testing.assert_allclose(y.double().numpy(), x.double().numpy() @ _sylvester(128), rtol=0, atol=2e-4)
+    for r in range(3):
+        assert np.array_equal(y[0, r].numpy(), _scalar_fwht(x[0, r].numpy()))
+    # orthogonal up to the factor D: dot products are preserved, applying it twice gives D * x
+    a, b = _rand((128,), 1, torch.float32), _rand((128,), 2, torch.float32)
+    assert abs(float(qr.fwht_ref(a) @ qr.fwht_ref(b)) / 128 - float(a @ b)) < 1e-4
+    torch.testing.assert_close(qr.fwht_ref(qr.fwht_ref(x)) / 128, x, rtol=1e-5, atol=1e-5)
+    # a lone outlier is spread evenly: |y| == |x_d| on every channel
+    e = torch.zeros(128)
+    e[37] = 20.0
+    assert (qr.fwht_ref(e).abs() == 20.0).all()
+
+
+# ------------------------------------------------------------------ int8 block quantizer
+@pytest.mark.parametrize("L", [5, 128, 130])
+def test_quant_q_matches_scalar_implementation(L):
+    D, sm = 8, 8**-0.5
+    q = _rand((1, L, 2, D), 20 + L, std=2.0)
+    qi, qs = qr.quant_q_ref(q, sm)
+    assert qi.shape == (1, 2, L, D) and qs.shape == (1, 2, L)  # one scale per query row
+    c = f32(f32(f32(sm) * f32(qr.LOG2E)) * f32(1.0 / D))
+    assert float(c) == qr.q_premul(sm, D).item()
+    for h in range(2):
+        rows = q[0, :, h].float().numpy()
+        x = np.stack([_scalar_fwht(r) * c for r in rows]).astype(np.float32)
+        ei, es = _scalar_block_int8(x, 1)
+        assert np.array_equal(qi[0, h].numpy(), ei)
+        assert np.array_equal(qs[0, h].numpy(), es)
+
+
+@pytest.mark.parametrize("L", [3, 64, 65, 200])
+def test_quant_k_matches_scalar_implementation(L):
+    D = 8
+    k = _rand((1, L, 2, D), 30 + L, std=1.0) + _rand((1, 1, 2, D), 99, std=2.0)
+    ki, ks, km = qr.quant_k_ref(k)
+    assert torch.equal(km, qr.k_mean_ref(k))
+    for h in range(2):
+        sm = (k[0, :, h].float().numpy() - km[0, h].float().numpy()[None, :]).astype(np.float32)
+        x = np.stack([_scalar_fwht(r) for r in sm])
+        ei, es = _scalar_block_int8(x, qr.BLKK)
+        assert np.array_equal(ki[0, h].numpy(), ei)
+        assert np.array_equal(ks[0, h].numpy(), es)
+    ki0, ks0, km0 = qr.quant_k_ref(k, smooth_k=False)
+    assert torch.count_nonzero(km0) == 0
+    ei, es = _scalar_block_int8(np.stack([_scalar_fwht(r) for r in k[0, :, 0].float().numpy()]), qr.BLKK)
+    assert np.array_equal(ki0[0, 0].numpy(), ei)
+
+
+def test_quant_hand_computed_blocks():
+    D = 4  # H4 rows: [1,1,1,1], [1,-1,1,-1], [1,1,-1,-1], [1,-1,-1,1]
+    # a row of equal values v transforms to (4v, 0, 0, 0): one entry 127, scale 4v/127
+    x = torch.full((1, 64, 1, D), 2.0, dtype=torch.bfloat16)
+    xi, xs, _ = qr.quant_k_ref(x, smooth_k=False)
+    assert (xi[..., 0] == 127).all() and (xi[..., 1:] == 0).all() and xs.item() == float(f32(8.0) / f32(127.0))
+    # smoothing removes a constant column entirely -> zero block: zeros and scale 0
+    xi, xs, km = qr.quant_k_ref(x, smooth_k=True)
+    assert (xi == 0).all() and xs.item() == 0.0 and (km == 2.0).all()
+    # exact ties after the transform.  rows (a,b,c,d) -> (a+b+c+d, a-b+c-d, a+b-c-d, a-b-c+d)
+    # (64, 63, 0, 0) -> (127, 1, 127, 1); (1, 0.5, 0, 0) -> (1.5, 0.5, 1.5, 0.5); (-2, -0.5, 0, 0) -> (-2.5,-1.5,-2.5,-1.5)
+    x = torch.tensor([[64.0, 63.0, 0, 0], [1.0, 0.5, 0, 0], [-2.0, -0.5, 0, 0]], dtype=torch.bfloat16).view(1, 3, 1, 4)
+    xi, xs, _ = qr.quant_k_ref(x, smooth_k=False)
+    assert xs.item() == 1.0  # amax 127 -> inv 1: values are rounded as they stand, half to even
+    assert xi[0, 0].tolist() == [[127, 1, 127, 1], [2, 0, 2, 0], [-2, -2, -2, -2]]
+    # a x20 outlier entry no longer dictates the step of its block: it is spread over the channels
+    x = torch.ones((1, 128, 1, D), dtype=torch.bfloat16)
+    x[0, 3, 0, 1] = -20.0
+    xi, xs, _ = qr.quant_k_ref(x, smooth_k=False)
+    # row 3 = (1,-20,1,1) -> (-17, 21, -21, 21); other rows -> (4,0,0,0); block amax 21
+    inv = f32(f32(127.0) / f32(21.0))
+    assert xi[0, 0, 3].tolist() == [int(np.rint(f32(v) * inv)) for v in (-17, 21, -21, 21)]
+    assert xi[0, 0, 0].tolist() == [int(np.rint(f32(4.0) * inv)), 0, 0, 0]
+    assert xs[0, 0].tolist() == [float(f32(21.0) / f32(127.0)), float(f32(4.0) / f32(127.0))]
+    # ragged tail: last block's scale comes from its valid rows only
+    x = torch.ones((1, 70, 1, D), dtype=torch.bfloat16)
+    x[0, 64:, 0, :] = 0.25
+    xi, xs, _ = qr.quant_k_ref(x, smooth_k=False)
+    assert xs.shape == (1, 1, 2) and (xi[0, 0, 64:, 0] == 127).all() and xs[0, 0, 1].item() == float(f32(1.0) / f32(127.0))
+    # Q: one scale per row, carries sm_scale * log2(e) / D
+    q = torch.tensor([[3.0, 3.0, 3.0, 3.0], [0.0, 0.0, 0.0, 0.0], [1.0, 0.0, 0.0, 0.0]], dtype=torch.bfloat16).view(1, 3, 1, 4)
+    qi, qs = qr.quant_q_ref(q, 0.25)
+    c = f32(f32(f32(0.25) * f32(qr.LOG2E)) * f32(0.25))
+    assert qs[0, 0].tolist() == [float(f32(f32(12.0) * c) / f32(127.0)), 0.0, float(f32(f32(1.0) * c) / f32(127.0))]
+    assert qi[0, 0].tolist() == [[127, 0, 0, 0], [0, 0, 0, 0], [127, 127, 127, 127]]
+
+
+def test_quant_invariants_on_workload_like_data():
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn((1, 1000, 2, 128), generator=g) + 2.0 * torch.randn((1, 1, 2, 128), generator=g)
+    mask = torch.rand(k.shape, generator=g) < 1e-3
+    k = torch.where(mask, k * 20, k).to(torch.bfloat16)
+    ki, ks, km = qr.quant_k_ref(k)
+    x = qr.fwht_ref(k.permute(0, 2, 1, 3).float() - km.float()[:, :, None])
+    s_row = ks.repeat_interleave(qr.BLKK, dim=2)[:, :, :1000, None]
+    err = (x - ki.float() * s_row).abs()
+    assert (err <= s_row * 0.5 * (1 + 1e-5)).all()
+    blocks = torch.cat([ki, ki.new_zeros(1, 2, 24, 128)], 2).view(1, 2, 16, -1)
+    assert (blocks.abs().amax(-1) == 127).all()
+    qi, qs = qr.quant_q_ref(k, 128**-0.5)
+    assert (qi.abs().amax(-1) == 127).all() and qs.shape == (1, 2, 1000)
+    # the int8 dot products reproduce q.(k - km) * sm_scale * log2(e)
+    s_int = qi[0, 0].float() @ ki[0, 0].float().t()
+    s = s_int * qs[0, 0][:, None] * s_row[0, 0, :, 0][None, :]
+    exact = (k[0, :, 0].double() @ (k[0, :, 0].double() - km[0, 0].double()).t()) * (128**-0.5 * qr.LOG2E)
+    assert (s.double() - exact).abs().max() < 0.02 * exact.abs().max()
+
+
+# ------------------------------------------------------------------ fp8 V
+def test_e4m3fn_cast_matches_format_definition():
+    table = qr.e4m3fn_decode_table()
+    codes = torch.arange(256, dtype=torch.uint8)
+    decoded = codes.view(torch.float8_e4m3fn).double()
+    finite = ~torch.isnan(table)
+    assert torch.equal(decoded[finite], table[finite]) and torch.isnan(decoded[~finite]).all()
+    assert table[finite].max() == 448.0 and table[1] == 2.0**-9
+    # round trip of every finite code is exact, so the cast is the identity on the grid
+    vals = table[finite].float()
+    back = vals.to(torch.float8_e4m3fn).float()
+    assert torch.equal(back, vals)
+    # nearest-even between grid points: brute force against the table
+    g = torch.Generator().manual_seed(3)
+    x = (torch.rand(4000, generator=g) * 2 - 1) * 448.0
+    x = torch.cat([x, x * 1e-2, x * 1e-4])
+    got = x.to(torch.float8_e4m3fn).double()
+    grid = table[finite]
+    dist = (x.double()[:, None] - grid[None, :]).abs()
+    best = dist.min(dim=1).values
+    assert torch.allclose((got - x.double()).abs(), best, rtol=0, atol=0)
+
+
+def test_quant_v_properties():
+    v = _rand((1, 333, 2, 16), 44, std=1.5)
+    v8, vs = qr.quant_v_ref(v)
+    assert v8.dtype == torch.float8_e4m3fn and v8.shape == (1, 2, 333, 16) and vs.shape == (1, 2, 16)
+    amax = v.float().abs().amax(dim=1)
+    assert torch.equal(vs, amax / torch.full_like(amax, 448.0))
+    assert (v8.float().abs().amax(dim=2) == 448.0).all()  # the channel max lands on +-448 exactly
+    deq = v8.float() * vs[:, :, None, :]
+    x = v.permute(0, 2, 1, 3).float()
+    assert ((deq - x).abs() <= x.abs() * 2**-4 + vs[:, :, None, :] * 2**-9).all()  # 3 mantissa bits
+    # scalar second implementation on one channel
+    table = qr.e4m3fn_decode_table()
+    grid = table[~torch.isnan(table)].numpy()
+    col = v[0, :, 1, 5].float().numpy()
+    a = f32(np.abs(col).max())
+    inv = f32(f32(448.0) / a)
+    for r in range(0, 333, 7):
+        y = float(f32(col[r] * inv))
+        y = max(-448.0, min(448.0, y))
+        d = np.abs(grid - y)
+        assert abs(float(v8[0, 1, r, 5].float()) - y) == d.min()
+    z = torch.zeros((1, 5, 1, 4), dtype=torch.bfloat16)
+    z8, zs = qr.quant_v_ref(z)
+    assert (z8.float() == 0).all() and (zs == 0).all()
+
+
+# ------------------------------------------------------------------ emulation of the fused kernel
+def _cos(a, b):
+    a, b = a.double().flatten(), b.double().flatten()
+    return float((a @ b) / (a.norm() * b.norm()))
+
+
+def test_sage_emul_close_to_sdpa_and_invariants():
+    B, L, H, D = 1, 300, 2, 128
+    q, v = _rand((B, L, H, D), 1), _rand((B, L, H, D), 3)
+    k = (_rand((B, L, H, D), 2).float() + 2.0 * _rand((1, 1, H, D), 4).float()).to(torch.bfloat16)
+    ref = sdpa_ref(q, k, v)
+    out = sage_emul_ref(q, k, v)
+    assert out.shape == ref.shape and out.dtype == ref.dtype
+    # the scheme's own error is ~3.5 % rms of |O| (two e4m3 roundings per product): cos-sim clears
+    # 0.999 at every length, while the ABSOLUTE error shrinks with |O| ~ 1/sqrt(L) - at L = 300 it
+    # is still above the 2e-2 that holds from the shortest measured workload (L = 1560) on.
+    assert _cos(out, ref) > 0.999 and (out.float() - ref.float()).abs().max() < 4e-2
+    # smoothing matters: without it the same data is visibly worse, never better by much
+    rough = sage_emul_ref(q, k, v, smooth_k=False)
+    assert (rough.float() - ref.float()).abs().mean() > (out.float() - ref.float()).abs().mean()
+    # rows of P sum to one: V == 1 gives O == 1 up to bf16/fp8 rounding of the normaliser
+    ones = torch.ones_like(v)
+    o1 = sage_emul_ref(q, k, ones).float()
+    assert (o1 - 1.0).abs().max() < 0.04
+    # permuting the keys inside a 64-key scale block permutes nothing in the output
+    perm = torch.cat([torch.randperm(64, generator=torch.Generator().manual_seed(9)) + 64 * i for i in range(4)] + [torch.arange(256, 300)])
+    o_perm = sage_emul_ref(q, k[:, perm], v[:, perm])
+    assert (o_perm.float() - out.float()).abs().max() < 4e-2
+    # GQA and rectangular shapes
+    kk, vv = k[:, :100, :1], v[:, :100, :1]
+    o_r = sage_emul_ref(q, kk, vv)
+    assert _cos(o_r, sdpa_ref(q, kk, vv)) > 0.999
+
+
+def test_sage_emul_meets_stated_tolerance_on_plumbing_workload():
+    """cos-sim >= 0.999 and max-abs <= 2e-2 against the SDPA oracle on the CPU-plumbing workload
+    (two of its 40 heads, full length 1560)."""
+    from ksanadit_amd.workloads import make_inputs
+
+    q, k, v = make_inputs("cpu_plumbing", heads=2)
+    ref, out = sdpa_ref(q, k, v), sage_emul_ref(q, k, v)
+    assert _cos(out, ref) >= 0.999
+    assert (out.float() - ref.float()).abs().max() <= 2e-2
+
+
+def test_sage_emul_survives_outliers():
+    """0.1 % entries x20 in Q and K (the headline workload's distribution, shortened): the
+    Hadamard stage plus per-token Q scales keep cos-sim >= 0.999."""
+    from ksanadit_amd.workloads import make_inputs
+
+    q, k, v = make_inputs("wan14b_480p", heads=1, seq=2048)
+    ref, out = sdpa_ref(q, k, v), sage_emul_ref(q, k, v)
+    assert _cos(out, ref) >= 0.999

@@ -1,0 +1,112 @@
+"""Bit-exact parity of the HIP quantizer (through the C ABI) with the CPU oracle."""
+
+import pytest
+import torch
+
+from ksanadit_amd import sage_ops
+from ksanadit_amd.layout import untile_k, untile_v
+from ksanadit_amd.workloads import make_inputs
+from oracle import quant_ref as qr
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_quant(q, k, v, dev, sm_scale=None, smooth_k=True):
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    ws = sage_ops.workspace_for(qd, kd)
+    ws.blob.fill_(0xA5)  # stale bytes must not leak into any output the attention kernel reads
+    sm_scale = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
+    sage_ops.quant_q(qd, ws, sm_scale)
+    sage_ops.quant_k(kd, ws, smooth_k)
+    sage_ops.quant_v(vd, ws)
+    torch.cuda.synchronize()
+    return ws
+
+
+def _check_against_oracle(q, k, v, dev, sm_scale=None, smooth_k=True):
+    ws = _run_quant(q, k, v, dev, sm_scale, smooth_k)
+    Lq, Lk = q.shape[1], k.shape[1]
+    sm = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
+    qi, qs = qr.quant_q_ref(q, sm)
+    ki, ks, km = qr.quant_k_ref(k, smooth_k=smooth_k)
+    v8, vs = qr.quant_v_ref(v)
+    got_qi = ws.q_i8.cpu()
+    assert torch.equal(got_qi[:, :, :Lq], qi), "q_int8 differs"
+    assert torch.count_nonzero(got_qi[:, :, Lq:]) == 0, "q padding rows not zero"
+    assert torch.equal(ws.q_scale.cpu()[:, :, :Lq], qs), "q_scale differs"
+    assert torch.equal(ws.k_mean.cpu(), km.float()), "k_mean differs"
+    k_tiles = ws.k_tiles.cpu()
+    assert torch.equal(untile_k(k_tiles, Lk), ki), "k_int8 differs"
+    nkb = k_tiles.shape[2]
+    if nkb * 64 > Lk:
+        full = untile_k(k_tiles, nkb * 64)
+        assert torch.count_nonzero(full[:, :, Lk:]) == 0, "k padding rows not zero"
+    assert torch.equal(ws.k_scale.cpu(), ks), "k_scale differs"
+    assert torch.equal(ws.v_scale.cpu(), vs), "v_scale differs"
+    v_tiles = ws.v_tiles.cpu()
+    assert torch.equal(untile_v(v_tiles, Lk), v8.view(torch.uint8)), "v_fp8 differs"
+    if nkb * 64 > Lk:
+        full = untile_v(v_tiles, nkb * 64)
+        assert torch.count_nonzero(full[:, :, Lk:]) == 0, "v padding rows not zero"
+
+
+def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, Lq, Hq, 128), generator=g)
+    k = torch.randn((B, Lk, Hkv, 128), generator=g) + 2.0 * torch.randn((1, 1, Hkv, 128), generator=g)
+    v = torch.randn((B, Lk, Hkv, 128), generator=g) * 1.5
+    return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+@pytest.mark.parametrize(
+    "B,Lq,Lk,Hq,Hkv",
+    [(1, 1, 1, 1, 1), (1, 100, 100, 2, 2), (2, 333, 77, 3, 3), (1, 128, 64, 2, 1), (1, 257, 513, 4, 2), (1, 640, 1000, 1, 1)],
+)
+def test_quantizer_bit_exact_small(hip_device, B, Lq, Lk, Hq, Hkv):
+    print(f"case B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv}", flush=True)
+    q, k, v = _rand_qkv(B, Lq, Lk, Hq, Hkv, seed=Lq * 7 + Lk)
+    _check_against_oracle(q, k, v, hip_device)
+
+
+def test_quantizer_bit_exact_fp16_and_options(hip_device):
+    q, k, v = _rand_qkv(1, 200, 300, 2, 2, seed=5, dtype=torch.float16)
+    _check_against_oracle(q, k, v, hip_device)
+    _check_against_oracle(q, k, v, hip_device, smooth_k=False)
+    _check_against_oracle(q, k, v, hip_device, sm_scale=0.37)
+
+
+def test_quantizer_edge_values(hip_device):
+    q, k, v = _rand_qkv(1, 130, 130, 2, 2, seed=9)
+    q[:, :3] = 0  # all-zero query rows -> scale 0, zeros
+    k[:, 64:128, 0] = k[:, 64:65, 0]  # a K block constant along the sequence ...
+    k[:, :, 1] = 1.25  # ... and a head that smoothing cancels completely
+    v[:, :, 0, 5] = 0  # a zero V channel
+    v[:, 7, 1, 9] = 300.0  # a lone huge V entry sets its channel's scale
+    q[0, 50, 1, 3] = 2.0**-120  # tiny magnitudes stay finite
+    _check_against_oracle(q, k, v, hip_device)
+    # exact .5 ties after scaling: a row (64, 63, 0, ...) transforms to +-127 / +-1 entries
+    q2 = torch.zeros_like(q)
+    q2[..., 0], q2[..., 1] = 64.0, 63.0
+    _check_against_oracle(q2, k, v, hip_device, sm_scale=1.0)
+
+
+def test_quantizer_strided_inputs(hip_device):
+    """q/k/v as views into one fused projection output, the way the DiT blocks produce them
+    (ksana/models/wan/wan_model.py:163-166): row stride 3*H*D, not contiguous."""
+    g = torch.Generator().manual_seed(3)
+    fused = torch.randn((2, 150, 3, 2, 128), generator=g).to(torch.bfloat16)
+    q, k, v = fused[:, :, 0], fused[:, :, 1], fused[:, :, 2]
+    assert not q.is_contiguous()
+    _check_against_oracle(q, k, v, hip_device)
+
+
+@pytest.mark.parametrize(
+    "name,heads,seq",
+    [("cpu_plumbing", None, None), ("wan5b_720p", 1, None), ("wan14b_480p", 2, None), ("wan14b_720p", 1, None), ("qwen_cfg", 4, None)],
+)
+def test_quantizer_bit_exact_workloads(hip_device, name, heads, seq):
+    """The five measured shapes at full sequence length (heads reduced where the CPU oracle
+    would otherwise take minutes; heads are independent in every stage)."""
+    print(f"workload {name} heads={heads}", flush=True)
+    q, k, v = make_inputs(name, heads=heads, seq=seq)
+    _check_against_oracle(q, k, v, hip_device)
