@@ -9,7 +9,8 @@ v_scale):
     P  = exp2(S - rowmax(S) + P_SHIFT)              Q already carries sm_scale * log2(e)
     O  = (fp8(P) . V_fp8) * v_scale / rowsum(P)
 
-It uses a full (not online) softmax in fp32, so it separates "error of the quantised
+It mirrors the kernel's tile-by-tile online softmax in fp32 (or, with ``online=False``, a
+full softmax), so it separates "error of the quantised
 scheme" from "bug in the kernel": the HIP kernel must agree with this far more tightly than
 either agrees with SDPA.  It is an approximation of SDPA by construction and is pinned by
 its distance to ``sdpa_ref`` plus exact invariants (see tests/test_oracle.py).
@@ -26,8 +27,13 @@ from .quant_ref import BLKK, BLKQ, FP8_MAX, quant_k_ref, quant_q_ref, quant_v_re
 P_SHIFT = 8.0
 
 
-def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False):
-    """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``."""
+def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True):
+    """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
+
+    ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
+    decides where each P lands on the e4m3 grid, so the fp8 rounding of P matches the kernel's
+    (a full softmax rounds P relative to the FINAL max - same accuracy, different bits).
+    """
     B, H, Lq, D = q_i8.shape
     Hkv, Lk = k_i8.shape[1], k_i8.shape[2]
     g = H // Hkv
@@ -43,20 +49,36 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
             if causal:
                 mask = torch.ones(Lq, Lk, dtype=torch.bool).tril(diagonal=Lk - Lq)
                 s = s.masked_fill(~mask, float("-inf"))
-            m = s.amax(dim=1, keepdim=True)
-            p = torch.exp2(s - m + P_SHIFT)
-            l = p.sum(dim=1, keepdim=True)
-            p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
-            o = (p8 @ v_fp8[b, hk].float()) * v_scale[b, hk][None, :] / l
+            vf = v_fp8[b, hk].float()
+            if online:
+                m = torch.full((Lq, 1), float("-inf"))
+                l = torch.zeros(Lq, 1)
+                acc = torch.zeros(Lq, D)
+                for j0 in range(0, Lk, BLKK):
+                    st = s[:, j0 : j0 + BLKK]
+                    m_new = torch.maximum(m, st.amax(dim=1, keepdim=True))
+                    alpha = torch.exp2(m - m_new)
+                    p = torch.exp2(st - m_new + P_SHIFT)
+                    l = l * alpha + p.sum(dim=1, keepdim=True)
+                    p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                    acc = acc * alpha + p8 @ vf[j0 : j0 + BLKK]
+                    m = m_new
+                o = acc / l * v_scale[b, hk][None, :]
+            else:
+                m = s.amax(dim=1, keepdim=True)
+                p = torch.exp2(s - m + P_SHIFT)
+                l = p.sum(dim=1, keepdim=True)
+                p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                o = (p8 @ vf) * v_scale[b, hk][None, :] / l
             out[b, :, h, :] = o.to(out_dtype)
     return out
 
 
-def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False):
+def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True):
     """[B, L, H, D] half in, same out: quantise with the oracle quantizer, then emulate."""
     D = q.shape[-1]
     sm_scale = D**-0.5 if sm_scale is None else sm_scale
     q_i8, q_scale = quant_q_ref(q, sm_scale)
     k_i8, k_scale, _ = quant_k_ref(k, smooth_k=smooth_k)
     v_fp8, v_scale = quant_v_ref(v)
-    return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal)
+    return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal, online=online)

@@ -57,8 +57,12 @@ def test_attention_vs_oracles_small(hip_device, B, Lq, Lk, Hq, Hkv):
     #    rescaling and the final bf16 rounding differ -> tight
     emul = _emul_from_ws(ws, Lq, Lk, q.dtype)
     scale = max(emul.float().abs().max().item(), 1e-3)
-    assert (out.float() - emul.float()).abs().max() <= 2e-2 * scale
-    assert _cos(out, emul) > 0.99995
+    diff = (out.float() - emul.float()).abs()
+    # an exp2 that lands within an ulp of an e4m3 rounding boundary may round the other way
+    # (6 % of one P): allowed on a handful of outputs, everything else agrees to bf16 rounding
+    assert diff.max() <= 2e-2 * scale
+    assert (diff > 1e-2 * scale * 0.5).float().mean() <= 1e-3
+    assert _cos(out, emul) > 0.99999
     # 2. vs SDPA: the scheme's own error dominates.  Short sequences give |O| ~ 0.1-1, so the
     #    absolute bound scales with the output magnitude here (2e-2 absolute holds from L=1560 on).
     ref = sdpa_ref(q, k, v)
