@@ -1,0 +1,163 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized attention path on one MI355X.
+
+A step is one full pass of the path over one batch of synthetic q/k/v already resident in HBM:
+quantize Q, quantize K (mean, Hadamard, int8), quantize V (fp8), fused attention - the same
+kernel sequence ``ksana_sage_forward`` enqueues, issued stage by stage so HIP events on the
+launch stream can bracket the attention kernel inside the timed region.
+
+Prints ONE JSON line.  ``value`` is attention flops (4*B*H*L^2*D) per second of whole-step time.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+METRIC = "Sage-attn effective TFLOPS & % INT8/FP8 MFMA peak, Wan-14B 480p (L=32760)"
+MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense INT8 (POP/s) = dense FP8 (PFLOP/s) = 5.0e15 /s
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=None, help="one of ksanadit_amd.workloads.WORKLOADS (default: headline)")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
+    return ap.parse_args()
+
+
+def cpu_baseline(workload, target_s: float):
+    """The oracle's SDPA (ksana/operations/attention/backends/sdpa.py:47-79 restated) on the host
+    cores, on a head-subsample of the same workload sized to about ``target_s`` seconds."""
+    from ksanadit_amd.workloads import make_inputs
+    from oracle.sdpa_ref import sdpa_ref
+
+    cores = torch.get_num_threads()
+    per_head = workload.flops / workload.H
+
+    def timed(heads, seq=None):
+        q, k, v = make_inputs(workload, heads=heads, seq=seq)
+        t0 = time.perf_counter()
+        sdpa_ref(q, k, v)
+        return time.perf_counter() - t0
+
+    probe_seq = min(workload.L, 4096)
+    timed(1, probe_seq)  # warm the thread pool
+    t_probe = timed(1, probe_seq)
+    rate = 4.0 * workload.B * probe_seq * probe_seq * workload.D / t_probe
+    heads = int(max(1, min(workload.H, target_s * rate / per_head)))
+    t = timed(heads)
+    flops = per_head * heads
+    return {
+        "value": round(flops / t / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{workload.name}: {heads} of {workload.H} heads at full L={workload.L}, bf16, one call, {t:.2f} s",
+        "ms_per_call_extrapolated": round(t / heads * workload.H * 1e3, 1),
+    }
+
+
+def main() -> int:
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (every run here has exactly one MI355X)", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 2
+
+    from ksanadit_amd import sage_ops
+    from ksanadit_amd.workloads import HEADLINE, WORKLOADS, make_inputs
+
+    w = WORKLOADS[args.workload or HEADLINE]
+    dev = torch.device("cuda:0")
+    q, k, v = make_inputs(w, device=dev)
+    ws = sage_ops.workspace_for(q, k)
+    out = torch.empty_like(q)
+    sm_scale = w.D**-0.5
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        sage_ops.quant_q(q, ws, sm_scale)
+        sage_ops.quant_k(k, ws, True)
+        sage_ops.quant_v(v, ws)
+        if ev:
+            ev[1].record()
+        sage_ops.attn_fwd(ws, out)
+        if ev:
+            ev[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for ev in events:
+        step(ev)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    ms_step = (t1 - t0) * 1e3 / args.steps
+    quant_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    attn_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    attn_tflops = w.flops / (attn_ms * 1e-3) / 1e12
+    n = w.elements
+    quant_bytes = 9.0 * n  # q, k, v read once as 16-bit, written once as 8-bit
+    quant_gbs = quant_bytes / (quant_ms * 1e-3) / 1e9
+
+    rec = {
+        "metric": METRIC,
+        "value": round(w.flops / (ms_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8+fp8",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: B={w.B} H={w.H} L={w.L} D={w.D} bf16 non-causal, seed {w.seed}"},
+        "attn_kernel_ms": round(attn_ms, 4),
+        "attn_kernel_tflops": round(attn_tflops, 2),
+        "pct_mfma_peak": round(100.0 * attn_tflops / MFMA_PEAK_TFLOPS, 2),
+        "quantizer_ms": round(quant_ms, 4),
+        "roofline": {
+            "kernel": "sage_attn_fwd_kernel",
+            "bound": "mfma",
+            "achieved": round(attn_tflops, 2),
+            "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(attn_tflops / MFMA_PEAK_TFLOPS, 4),
+            "traffic": None,
+        },
+        "quantizer_roofline": {
+            "kernels": "col_partial x2, finalize x2, quant_q, quant_k, quant_v",
+            "bound": "hbm",
+            "achieved": round(quant_gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(quant_gbs / HBM_PEAK_GBS, 4),
+            "algorithmic_bytes": quant_bytes,
+        },
+    }
+    if args.cpu_seconds > 0:
+        rec["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
+    print(json.dumps(rec))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

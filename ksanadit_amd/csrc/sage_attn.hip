@@ -3,7 +3,7 @@
 //
 // Work split.  One workgroup = 8 waves = 256 query rows of one (batch, head); each wave owns
 // 32 query rows for the whole key loop.  Keys are consumed in tiles of 64 rows (= one int8
-// K scale block; Q scales are per row, i.e. per lane), K and V^T tiles are staged in LDS (double buffered) and shared by the 8 waves.
+// K scale block; Q scales are per row, i.e. per lane), K and V^T tiles are staged in a 3-deep LDS ring shared by the 8 waves.
 // Two waves share a SIMD, so one wave's softmax (VALU) overlaps the other's MFMAs.
 //
 // Fragment algebra (32x32 MFMA, lane l: l32 = l % 32, hh = l / 32):
@@ -39,6 +39,7 @@ constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f
 constexpr float kMagicF = 12582912.0f;
 constexpr float kPShift = 8.0f;           // P is scaled by 2^8 before the e4m3 cast
 constexpr int kStageBytes = 2 * kTileBytes;  // K tile + V tile
+constexpr int kStages = 3;                   // LDS ring: tile j (V), j+1 (K), j+2 (in flight)
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -57,6 +58,21 @@ __device__ __forceinline__ void store4(uint16_t* dst, float a, float b, float c,
     hi = __builtin_bit_cast(uint32_t, y);
   }
   *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+}
+
+// S^T tile (64 keys x 32 queries) of one wave: two 32-key sub-tiles, four 32-channel steps.
+__device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const v4i (&qf)[4], const v16i& magic,
+                                        v16i (&acc)[2]) {
+  acc[0] = magic;
+  acc[1] = magic;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const v4i kf = *reinterpret_cast<const v4i*>(k_stage + ((t * 4 + s) * 64 + lane) * 16);
+      acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], acc[t], 0, 0, 0);
+    }
+  }
 }
 
 template <int DT>
@@ -98,7 +114,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
   float m_run = -INFINITY;  // running row max (log2 domain) of query l32
-  float l_run = 0.0f;       // this lane's share of the running row sum
+  float l_part[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // this lane's share of the running row sum
 
   v16i magic;
 #pragma unroll
@@ -107,118 +123,161 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const uint8_t* k_src = reinterpret_cast<const uint8_t*>(p.k_tiles) + (int64_t)bhk * p.nkb * kTileBytes + tid * 16;
   const uint8_t* v_src = p.v_tiles + (int64_t)bhk * p.nkb * kTileBytes + tid * 16;
   const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb;
+  const int nkb = p.nkb;
 
-  // ---- prologue: tile 0 -> LDS stage 0 -------------------------------------------------
-  {
-    const uint4 kreg = *reinterpret_cast<const uint4*>(k_src);
-    const uint4 vreg = *reinterpret_cast<const uint4*>(v_src);
-    *reinterpret_cast<uint4*>(smem + tid * 16) = kreg;
-    *reinterpret_cast<uint4*>(smem + kTileBytes + tid * 16) = vreg;
+  // ---- prologue: tiles 0 and 1 -> LDS stages 0 and 1; S^T of tile 0 --------------------
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (j < nkb) {
+      const uint4 kreg = *reinterpret_cast<const uint4*>(k_src + (int64_t)j * kTileBytes);
+      const uint4 vreg = *reinterpret_cast<const uint4*>(v_src + (int64_t)j * kTileBytes);
+      *reinterpret_cast<uint4*>(smem + j * kStageBytes + tid * 16) = kreg;
+      *reinterpret_cast<uint4*>(smem + j * kStageBytes + kTileBytes + tid * 16) = vreg;
+    }
   }
   __syncthreads();
 
-  for (int j = 0; j < p.nkb; ++j) {
-    const uint8_t* stage = smem + (j & 1) * kStageBytes;
-    const bool has_next = j + 1 < p.nkb;
-    uint4 kreg = make_uint4(0, 0, 0, 0), vreg = make_uint4(0, 0, 0, 0);
-    if (has_next) {
-      kreg = *reinterpret_cast<const uint4*>(k_src + (int64_t)(j + 1) * kTileBytes);
-      vreg = *reinterpret_cast<const uint4*>(v_src + (int64_t)(j + 1) * kTileBytes);
-    }
+  const bool has_tail = (p.Lk & (kBlkK - 1)) != 0;  // keys >= Lk live only in the last tile
+  const int n_main = has_tail ? nkb - 1 : nkb;       // tiles handled by the branch-free loop
 
-    if (active) {
-      // ---- S^T = K . Q^T : two 32-key sub-tiles, four 32-channel steps -------------
-      v16i acc[2] = {magic, magic};
+  // HBM -> registers for tile j+2 (clamped: the last two iterations re-fetch the last tile into
+  // a stage nobody reads any more, which keeps the loop body free of branches)
+  auto fetch = [&](int j, uint4& kreg, uint4& vreg) {
+    const int jl = min(j + 2, nkb - 1);
+    kreg = *reinterpret_cast<const uint4*>(k_src + (int64_t)jl * kTileBytes);
+    vreg = *reinterpret_cast<const uint4*>(v_src + (int64_t)jl * kTileBytes);
+  };
+  auto stash = [&](int j, const uint4& kreg, const uint4& vreg) {
+    uint8_t* dst = smem + ((j + 2) % kStages) * kStageBytes;
+    *reinterpret_cast<uint4*>(dst + tid * 16) = kreg;
+    *reinterpret_cast<uint4*>(dst + kTileBytes + tid * 16) = vreg;
+  };
+
+  if (!active) {
+    // same barrier sequence as the active waves, moving tiles only
+    for (int j = 0; j < n_main; ++j) {
+      uint4 kreg, vreg;
+      fetch(j, kreg, vreg);
+      stash(j, kreg, vreg);
+      __syncthreads();
+    }
+    return;
+  }
+
+  // running max update for one tile; rescales O and the row sum when the max of any row moved
+  auto update_max = [&](const v16i (&s_cur)[2], float sc) {
+    int imax = s_cur[0][0];
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const v4i kf = *reinterpret_cast<const v4i*>(stage + ((t * 4 + s) * 64 + lane) * 16);
-          acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], acc[t], 0, 0, 0);
-        }
-      }
-      const bool tail = j == p.nkb - 1 && (p.Lk & (kBlkK - 1)) != 0;  // keys >= Lk live only here
-      if (tail) {
+      for (int r = 0; r < 16; ++r) imax = max(imax, s_cur[t][r]);
+    {
+      // the other half of query l32's keys lives in lane l32 + 32
+      int other = imax;
+      const auto sw = __builtin_amdgcn_permlane32_swap(imax, other, false, false);
+      imax = max(sw[0], sw[1]);
+    }
+    const float m_tile = (float)(imax - kMagicI) * sc;
+    const float m_new = fmaxf(m_run, m_tile);
+    if (__any(m_new > m_run)) {
+      const float alpha = fast_exp2(m_run - m_new);
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+      for (int i = 0; i < 4; ++i) l_part[i] *= alpha;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = j * kBlkK + 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
-            if (key >= p.Lk) acc[t][r] = kMagicI - (1 << 22);  // below every real score
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+      m_run = m_new;
+    }
+  };
+  // P = exp2(sc*dot - m_run + shift) packed to e4m3 in MFMA operand order; the magic is folded
+  // into the constant, which is off by at most ~1.5 integer steps of the dot product
+  auto exp_and_pack = [&](const v16i (&s_cur)[2], float sc, v8i& pf, int j, auto is_tail) {
+    const float c = (kPShift - m_run) - kMagicF * sc;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          e[i] = fast_exp2(__builtin_fmaf(__int_as_float(s_cur[t][4 * g + i]), sc, c));
+          if constexpr (decltype(is_tail)::value) {
+            const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
+            if (key >= p.Lk) e[i] = 0.0f;
           }
-      }
-      const float sc = qs * ks_ptr[j];
-
-      // ---- online softmax ---------------------------------------------------------
-      int imax = acc[0][0];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) imax = max(imax, acc[t][r]);
-      imax = max(imax, __shfl_xor(imax, 32));
-      const float m_tile = (float)(imax - kMagicI) * sc;
-      const float m_new = fmaxf(m_run, m_tile);
-      if (__any(m_new > m_run)) {
-        const float alpha = fast_exp2(m_run - m_new);
-        l_run *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-        m_run = m_new;
-      }
-      // exponent of key r: sc*dot - m_run + shift, with the magic folded into the constant;
-      // the constant is off by at most ~1.5 integer steps of the dot product
-      const float c = (kPShift - m_run) - kMagicF * sc;
-      v8i pf;
-      auto exp_and_pack = [&](auto is_tail) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            float e[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              e[i] = fast_exp2(__builtin_fmaf(__int_as_float(acc[t][4 * g + i]), sc, c));
-              if constexpr (decltype(is_tail)::value) {
-                const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
-                if (key >= p.Lk) e[i] = 0.0f;
-              }
-              l_run += e[i];
-            }
-            int w = 0;
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], w, false);
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
-            pf[4 * t + g] = w;
-          }
+          l_part[i] += e[i];
         }
-      };
-      if (tail)
-        exp_and_pack(std::true_type{});
-      else
-        exp_and_pack(std::false_type{});
-      // ---- O^T += V^T . P^T -------------------------------------------------------
-      const uint8_t* vst = stage + kTileBytes;
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
-        const v4i hi = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 1) * 64 + lane) * 16);
-        const v8i vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[dt], 0, 0, 0, 0, 0, 0);
+        int w = 0;
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], w, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
+        pf[4 * t + g] = w;
       }
     }
-
-    if (has_next) {
-      uint8_t* nxt = smem + ((j + 1) & 1) * kStageBytes;
-      *reinterpret_cast<uint4*>(nxt + tid * 16) = kreg;
-      *reinterpret_cast<uint4*>(nxt + kTileBytes + tid * 16) = vreg;
+  };
+  // O^T += V^T . P^T
+  auto pv_tile = [&](const uint8_t* vst, const v8i& pf) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
+      const v4i hi = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 1) * 64 + lane) * 16);
+      const v8i vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[dt], 0, 0, 0, 0, 0, 0);
     }
+  };
+
+  v16i s_a[2], s_b[2];
+  qk_tile(smem, lane, qf, magic, s_a);
+
+  // One full key tile.  The S^T MFMAs of the NEXT tile sit in the same basic block as this
+  // tile's exponentials, so the scheduler can run them under the VALU work; the tile after
+  // that travels HBM -> registers -> LDS meanwhile (3-stage ring).
+  auto tile_step = [&](int j, v16i (&s_cur)[2], v16i (&s_nxt)[2]) {
+    uint4 kreg, vreg;
+    fetch(j, kreg, vreg);
+    const float sc = qs * ks_ptr[j];
+    update_max(s_cur, sc);
+    // stage (j+1)%3 holds tile j+1 (stale bytes after the last tile: computed, never used)
+    qk_tile(smem + ((j + 1) % kStages) * kStageBytes, lane, qf, magic, s_nxt);
+    v8i pf;
+    exp_and_pack(s_cur, sc, pf, j, std::false_type{});
+    pv_tile(smem + (j % kStages) * kStageBytes + kTileBytes, pf);
+    stash(j, kreg, vreg);
+    // interleave: one MFMA (32 cycles of matrix pipe) per ~14 VALU instructions
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read (K fragment)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, 14, 0);  // VALU (fma / exp2 / add / cvt)
+    }
+    // after this barrier: tile j+2 is visible, and nobody reads stage j%3 any more
     __syncthreads();
+  };
+
+  for (int j = 0; j < n_main; j += 2) {
+    tile_step(j, s_a, s_b);
+    if (j + 1 < n_main) tile_step(j + 1, s_b, s_a);
+  }
+  if (has_tail) {
+    const int j = nkb - 1;
+    v16i (&s_cur)[2] = (n_main & 1) ? s_b : s_a;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = j * kBlkK + 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (key >= p.Lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
+      }
+    const float sc = qs * ks_ptr[j];
+    update_max(s_cur, sc);
+    v8i pf;
+    exp_and_pack(s_cur, sc, pf, j, std::true_type{});
+    pv_tile(smem + (j % kStages) * kStageBytes + kTileBytes, pf);
   }
 
   // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
-  if (!active) return;
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float l_lane = (l_part[0] + l_part[1]) + (l_part[2] + l_part[3]);
+  const float l_tot = l_lane + __shfl_xor(l_lane, 32);
   const float inv_l = 1.0f / l_tot;
   const int q = q0 + l32;
   if (q < p.Lq) {
@@ -244,7 +303,7 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const int n_wg = p.B * p.Hq * n_qwg;
   const int wg_per_xcd = (n_wg + 7) / 8;
   const dim3 grid(wg_per_xcd * 8), block(kThreadsAttn);
-  const size_t lds = 2 * kStageBytes;
+  const size_t lds = kStages * kStageBytes;
   if (p.o.dtype == KSANA_SAGE_BF16)
     sage_attn_fwd_kernel<KSANA_SAGE_BF16><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   else
