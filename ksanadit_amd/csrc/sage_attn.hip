@@ -3,7 +3,7 @@
 //
 // Work split.  One workgroup = 8 waves = 256 query rows of one (batch, head); each wave owns
 // 32 query rows for the whole key loop.  Keys are consumed in tiles of 64 rows (= one int8
-// K scale block; Q scales are per row, i.e. per lane), K and V^T tiles are staged in a 3-deep LDS ring shared by the 8 waves.
+// K scale block; Q scales are per row, i.e. per lane), K and V^T tiles are copied asynchronously (global_load ... lds) into an 8-deep LDS ring shared by the 8 waves.
 // Two waves share a SIMD, so one wave's softmax (VALU) overlaps the other's MFMAs.
 //
 // Fragment algebra (32x32 MFMA, lane l: l32 = l % 32, hh = l / 32):
@@ -39,9 +39,18 @@ constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f
 constexpr float kMagicF = 12582912.0f;
 constexpr float kPShift = 8.0f;           // P is scaled by 2^8 before the e4m3 cast
 constexpr int kStageBytes = 2 * kTileBytes;  // K tile + V tile
-constexpr int kStages = 3;                   // LDS ring: tile j (V), j+1 (K), j+2 (in flight)
+constexpr int kStages = 8;                   // LDS ring (power of two): tiles j-1 .. j+kAhead live at step j
+constexpr int kAhead = 4;                    // HBM -> LDS copies are issued this many tiles ahead (<= 6)
+constexpr int kMaxKeyTiles = 4096;           // K scales of one head are kept in LDS: Lk <= 262144
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Opaque use+def at this program point: keeps the optimizer from sinking the computation of
+// `x` into a later basic block (it emits no instruction).
+template <typename T>
+__device__ __forceinline__ void pin(T& x) {
+  asm volatile("" : "+v"(x));
+}
 
 template <int DT>
 __device__ __forceinline__ void store4(uint16_t* dst, float a, float b, float c, float d) {
@@ -124,48 +133,57 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const uint8_t* v_src = p.v_tiles + (int64_t)bhk * p.nkb * kTileBytes + tid * 16;
   const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb;
   const int nkb = p.nkb;
+  // K scales live in LDS behind the ring: a per-tile global load would share the in-order
+  // vmcnt queue with the tile copies and stall on all of them
+  float* s_ks = reinterpret_cast<float*>(smem + kStages * kStageBytes);
+  for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
 
-  // ---- prologue: tiles 0 and 1 -> LDS stages 0 and 1; S^T of tile 0 --------------------
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    if (j < nkb) {
-      const uint4 kreg = *reinterpret_cast<const uint4*>(k_src + (int64_t)j * kTileBytes);
-      const uint4 vreg = *reinterpret_cast<const uint4*>(v_src + (int64_t)j * kTileBytes);
-      *reinterpret_cast<uint4*>(smem + j * kStageBytes + tid * 16) = kreg;
-      *reinterpret_cast<uint4*>(smem + j * kStageBytes + kTileBytes + tid * 16) = vreg;
-    }
-  }
-  __syncthreads();
-
+  // ---- asynchronous tile copies: HBM/L2 -> LDS without passing through registers ----------
+  // Each wave moves its 1 KiB slice of the K tile and of the V^T tile (lane i -> byte 16*i of
+  // the slice).  Copies retire in issue order, so "at most 2*n outstanding" == "all but the
+  // newest n tiles have landed".
   const bool has_tail = (p.Lk & (kBlkK - 1)) != 0;  // keys >= Lk live only in the last tile
-  const int n_main = has_tail ? nkb - 1 : nkb;       // tiles handled by the branch-free loop
+  const int n_main = has_tail ? nkb - 1 : nkb;       // tiles handled by the pipelined loop
+  auto issue_copy = [&](int tile) {
+    // clamped: past the end the last tile is copied again into a stage nobody reads any more,
+    // which keeps the loop free of branches and the outstanding-copy count constant
+    const int jl = min(tile, nkb - 1);
+    uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes + wave * 1024;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_src + (int64_t)jl * kTileBytes),
+                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_src + (int64_t)jl * kTileBytes),
+                                     (__attribute__((address_space(3))) void*)(dst + kTileBytes), 16, 0, 0);
+  };
+  // wait until every copy except those of the newest (kAhead - 2) tiles has landed, then meet
+  // the other waves.  Plain s_barrier: a fence here would drain ALL copies and undo the prefetch.
+  auto tile_barrier = [&]() {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * (kAhead - 2)) : "memory");
+  };
 
-  // HBM -> registers for tile j+2 (clamped: the last two iterations re-fetch the last tile into
-  // a stage nobody reads any more, which keeps the loop body free of branches)
-  auto fetch = [&](int j, uint4& kreg, uint4& vreg) {
-    const int jl = min(j + 2, nkb - 1);
-    kreg = *reinterpret_cast<const uint4*>(k_src + (int64_t)jl * kTileBytes);
-    vreg = *reinterpret_cast<const uint4*>(v_src + (int64_t)jl * kTileBytes);
-  };
-  auto stash = [&](int j, const uint4& kreg, const uint4& vreg) {
-    uint8_t* dst = smem + ((j + 2) % kStages) * kStageBytes;
-    *reinterpret_cast<uint4*>(dst + tid * 16) = kreg;
-    *reinterpret_cast<uint4*>(dst + kTileBytes + tid * 16) = vreg;
-  };
+  // Stage 7's V half is read (times P = 0) by the first loop iteration: make it finite.
+  *reinterpret_cast<uint4*>(smem + (kStages - 1) * kStageBytes + kTileBytes + tid * 16) = make_uint4(0, 0, 0, 0);
+#pragma unroll
+  for (int t = 0; t < kAhead; ++t) issue_copy(t);
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * (kAhead - 2)) : "memory");  // tiles 0, 1 visible
 
   if (!active) {
-    // same barrier sequence as the active waves, moving tiles only
+    // same copy / barrier sequence as the active waves
     for (int j = 0; j < n_main; ++j) {
-      uint4 kreg, vreg;
-      fetch(j, kreg, vreg);
-      stash(j, kreg, vreg);
-      __syncthreads();
+      issue_copy(j + kAhead);
+      tile_barrier();
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     return;
   }
 
-  // running max update for one tile; rescales O and the row sum when the max of any row moved
-  auto update_max = [&](const v16i (&s_cur)[2], float sc) {
+  auto scale_o = [&](float alpha) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+  };
+  // new running max of query l32 after the tile in s_cur; returns 2^(old max - new max)
+  auto update_max = [&](const v16i (&s_cur)[2], float sc) -> float {
     int imax = s_cur[0][0];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -179,86 +197,117 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     }
     const float m_tile = (float)(imax - kMagicI) * sc;
     const float m_new = fmaxf(m_run, m_tile);
-    if (__any(m_new > m_run)) {
-      const float alpha = fast_exp2(m_run - m_new);
+    const float alpha = fast_exp2(m_run - m_new);
+    m_run = m_new;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) l_part[i] *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-      m_run = m_new;
-    }
+    for (int i = 0; i < 4; ++i) l_part[i] *= alpha;
+    return alpha;
   };
-  // P = exp2(sc*dot - m_run + shift) packed to e4m3 in MFMA operand order; the magic is folded
-  // into the constant, which is off by at most ~1.5 integer steps of the dot product
-  auto exp_and_pack = [&](const v16i (&s_cur)[2], float sc, v8i& pf, int j, auto is_tail) {
-    const float c = (kPShift - m_run) - kMagicF * sc;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float e[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          e[i] = fast_exp2(__builtin_fmaf(__int_as_float(s_cur[t][4 * g + i]), sc, c));
-          if constexpr (decltype(is_tail)::value) {
-            const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
-            if (key >= p.Lk) e[i] = 0.0f;
-          }
-          l_part[i] += e[i];
-        }
-        int w = 0;
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], w, false);
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
-        pf[4 * t + g] = w;
-      }
-    }
-  };
-  // O^T += V^T . P^T
-  auto pv_tile = [&](const uint8_t* vst, const v8i& pf) {
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
-      const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
-      const v4i hi = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 1) * 64 + lane) * 16);
-      const v8i vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[dt], 0, 0, 0, 0, 0, 0);
-    }
+  // p = exp2(sc*dot - m_run + shift); the magic is folded into the constant c, which is off by
+  // at most ~1.5 integer steps of the dot product
+  auto p_of = [&](int acc_bits, float sc, float c) { return fast_exp2(__builtin_fmaf(__int_as_float(acc_bits), sc, c)); };
+  // O^T += V^T . P^T for one 32-channel slice
+  auto pv_slice = [&](const uint8_t* vst, int dt, const v8i& pf) {
+    const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
+    const v4i hi = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 1) * 64 + lane) * 16);
+    const v8i vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[dt], 0, 0, 0, 0, 0, 0);
   };
 
   v16i s_a[2], s_b[2];
   qk_tile(smem, lane, qf, magic, s_a);
 
-  // One full key tile.  The S^T MFMAs of the NEXT tile sit in the same basic block as this
-  // tile's exponentials, so the scheduler can run them under the VALU work; the tile after
-  // that travels HBM -> registers -> LDS meanwhile (3-stage ring).
+  // Software pipeline, one key tile per step.  While this tile's probabilities are computed on
+  // the VALU, the matrix pipe runs the S^T MFMAs of the NEXT tile and the PV MFMAs of the
+  // PREVIOUS tile: every MFMA below is followed by the VALU work that hides it, and
+  // sched_barrier pins that order.  Because PV lags one tile, so does the rescaling of O:
+  //   at step j   O holds tiles <= j-2 relative to max m(j-2); alpha_prev = 2^(m(j-2) - m(j-1))
+  //   step j      O *= alpha_prev (rare branch), then O += P(j-1) V(j-1), both relative to m(j-1)
+  // LDS ring of 8 stages: tile j-1 (V), j (V next step), j+1 (K), j+2 .. j+4 (arriving).
+  v8i pf_prev = {0, 0, 0, 0, 0, 0, 0, 0};
+  float alpha_prev = 1.0f;
   auto tile_step = [&](int j, v16i (&s_cur)[2], v16i (&s_nxt)[2]) {
-    uint4 kreg, vreg;
-    fetch(j, kreg, vreg);
-    const float sc = qs * ks_ptr[j];
-    update_max(s_cur, sc);
-    // stage (j+1)%3 holds tile j+1 (stale bytes after the last tile: computed, never used)
-    qk_tile(smem + ((j + 1) % kStages) * kStageBytes, lane, qf, magic, s_nxt);
+    issue_copy(j + kAhead);
+    const float sc = qs * s_ks[j];
+    if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
+    alpha_prev = update_max(s_cur, sc);
+    const float c = (kPShift - m_run) - kMagicF * sc;
+    const uint8_t* kst = smem + ((j + 1) & (kStages - 1)) * kStageBytes;
+    const uint8_t* vst = smem + ((j - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
     v8i pf;
-    exp_and_pack(s_cur, sc, pf, j, std::false_type{});
-    pv_tile(smem + (j % kStages) * kStageBytes + kTileBytes, pf);
-    stash(j, kreg, vreg);
-    // interleave: one MFMA (32 cycles of matrix pipe) per ~14 VALU instructions
+    // LDS operands are requested two MFMAs ahead of their use (12 fragments: 8 of K, 4 of V^T)
+    auto k_frag = [&](int i) { return *reinterpret_cast<const v4i*>(kst + (((i & 1) * 4 + (i >> 1)) * 64 + lane) * 16); };
+    auto v_frag = [&](int dt) {
+      const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
+      const v4i hi = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 1) * 64 + lane) * 16);
+      return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    v4i kf[3];
+    v8i vf[3];
+    kf[0] = k_frag(0);
+    kf[1] = k_frag(1);
+    __builtin_amdgcn_sched_barrier(0);
+    // 8 x [S^T MFMA of tile j+1 (32 matrix cycles) | 2 probabilities of tile j]
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read (K fragment)
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x002, 14, 0);  // VALU (fma / exp2 / add / cvt)
+      const int s = i >> 1, t = i & 1;
+      if (i + 2 < 8)
+        kf[(i + 2) % 3] = k_frag(i + 2);
+      else
+        vf[i + 2 - 8] = v_frag(i + 2 - 8);
+      s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i % 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
+      const float e0 = p_of(s_cur[0][2 * i], sc, c), e1 = p_of(s_cur[0][2 * i + 1], sc, c);
+      l_part[(2 * i) & 3] += e0;
+      l_part[(2 * i + 1) & 3] += e1;
+      if (i & 1) {
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, pf[i >> 1], true);
+        pin(w);
+        pf[i >> 1] = w;
+      } else {
+        pf[i >> 1] = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, 0, false);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // after this barrier: tile j+2 is visible, and nobody reads stage j%3 any more
-    __syncthreads();
+    // 4 x [PV MFMA of tile j-1 (64 matrix cycles) | 4 probabilities of tile j]
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      if (dt + 2 < 4) vf[(dt + 2) % 3] = v_frag(dt + 2);
+      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt % 3], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
+      float e[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        e[i] = p_of(s_cur[1][4 * dt + i], sc, c);
+        l_part[i] += e[i];
+      }
+      int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], 0, false);
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
+      pin(w);
+      pf[4 + dt] = w;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pin(l_part[i]);
+    pf_prev = pf;
+    // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
+    tile_barrier();
   };
 
-  for (int j = 0; j < n_main; j += 2) {
-    tile_step(j, s_a, s_b);
-    if (j + 1 < n_main) tile_step(j + 1, s_b, s_a);
+  {
+    int j = 0;
+    for (; j + 2 <= n_main; j += 2) {
+      tile_step(j, s_a, s_b);
+      tile_step(j + 1, s_b, s_a);
+    }
+    if (j < n_main) tile_step(j, s_a, s_b);
   }
-  if (has_tail) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may outlive the workgroup's LDS
+  if (n_main > 0) {  // drain: PV of the last pipelined tile
+    scale_o(alpha_prev);
+    const uint8_t* vst = smem + ((n_main - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_prev);
+  }
+  if (has_tail) {  // ragged last tile, not pipelined: mask keys >= Lk
     const int j = nkb - 1;
     v16i (&s_cur)[2] = (n_main & 1) ? s_b : s_a;
 #pragma unroll
@@ -268,11 +317,27 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         const int key = j * kBlkK + 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
         if (key >= p.Lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
       }
-    const float sc = qs * ks_ptr[j];
-    update_max(s_cur, sc);
+    const float sc = qs * s_ks[j];
+    scale_o(update_max(s_cur, sc));
+    const float c = (kPShift - m_run) - kMagicF * sc;
     v8i pf;
-    exp_and_pack(s_cur, sc, pf, j, std::true_type{});
-    pv_tile(smem + (j % kStages) * kStageBytes + kTileBytes, pf);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
+          e[i] = key < p.Lk ? p_of(s_cur[t][4 * g + i], sc, c) : 0.0f;
+          l_part[i] += e[i];
+        }
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], 0, false);
+        pf[4 * t + g] = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
+      }
+    const uint8_t* vst = smem + (j & (kStages - 1)) * kStageBytes + kTileBytes;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf);
   }
 
   // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
@@ -299,11 +364,22 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 }  // namespace
 
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
+  if (p.nkb > kMaxKeyTiles) return hipErrorInvalidValue;
   const int n_qwg = (p.Lq + kAttnQPerWg - 1) / kAttnQPerWg;
   const int n_wg = p.B * p.Hq * n_qwg;
   const int wg_per_xcd = (n_wg + 7) / 8;
   const dim3 grid(wg_per_xcd * 8), block(kThreadsAttn);
-  const size_t lds = kStages * kStageBytes;
+  // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
+  const size_t lds = kStages * kStageBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
+  // more than 64 KiB of dynamic LDS has to be requested per kernel, once
+  static const hipError_t attr_bf16 = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&sage_attn_fwd_kernel<KSANA_SAGE_BF16>), hipFuncAttributeMaxDynamicSharedMemorySize,
+      kStages * kStageBytes + kMaxKeyTiles * 4);
+  static const hipError_t attr_fp16 = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&sage_attn_fwd_kernel<KSANA_SAGE_FP16>), hipFuncAttributeMaxDynamicSharedMemorySize,
+      kStages * kStageBytes + kMaxKeyTiles * 4);
+  if (attr_bf16 != hipSuccess) return attr_bf16;
+  if (attr_fp16 != hipSuccess) return attr_fp16;
   if (p.o.dtype == KSANA_SAGE_BF16)
     sage_attn_fwd_kernel<KSANA_SAGE_BF16><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   else

@@ -30,6 +30,7 @@ int check_shape(const ksana_sage_shape* s) {
                 s->Hkv, s->Lq, s->Lk);
   if (s->Hq % s->Hkv != 0) return fail(KSANA_SAGE_EINVAL, "Hq=%d is not a multiple of Hkv=%d", s->Hq, s->Hkv);
   if (s->D != ksana_sage::kD) return fail(KSANA_SAGE_ENOTSUP, "head size %d not supported (only 128)", s->D);
+  if (s->Lk > 262144) return fail(KSANA_SAGE_ENOTSUP, "Lk=%d exceeds 262144 (K scales of one head are kept in LDS)", s->Lk);
   if ((int64_t)s->B * s->Hq > 65535 * 8 || s->Hq > 65535 || s->B > 65535)
     return fail(KSANA_SAGE_EINVAL, "B*H too large for the launch grid");
   return 0;
