@@ -97,7 +97,8 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const int b = bh / p.Hq, h = bh - b * p.Hq;
   const int bhk = b * p.Hkv + h / (p.Hq / p.Hkv);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction: keep it scalar
   const int l32 = lane & 31, hh = lane >> 5;
   const int q0 = qwg * kAttnQPerWg + wave * 32;
   const bool active = q0 < p.Lq;  // wave-uniform; inactive waves only help move tiles
@@ -123,7 +124,13 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
   float m_run = -INFINITY;  // running row max (log2 domain) of query l32
-  float l_part[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // this lane's share of the running row sum
+  // Row sums come from the matrix pipe too: an all-ones A operand (e4m3 1.0 = 0x38) makes every
+  // row of `lacc` the sum over keys of the SAME e4m3-rounded P the numerator uses.  Only
+  // register 0 is read (all 16 hold the same value), so only it is rescaled.
+  v16f lacc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) lacc[r] = 0.0f;
+  const v8i ones = {0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838};
 
   v16i magic;
 #pragma unroll
@@ -181,6 +188,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    lacc[0] *= alpha;
   };
   // new running max of query l32 after the tile in s_cur; returns 2^(old max - new max)
   auto update_max = [&](const v16i (&s_cur)[2], float sc) -> float {
@@ -199,8 +207,6 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const float m_new = fmaxf(m_run, m_tile);
     const float alpha = fast_exp2(m_run - m_new);
     m_run = m_new;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) l_part[i] *= alpha;
     return alpha;
   };
   // p = exp2(sc*dot - m_run + shift); the magic is folded into the constant c, which is off by
@@ -230,6 +236,8 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     issue_copy(j + kAhead);
     const float sc = qs * s_ks[j];
     if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
+    // row sums of tile j-1: 64 matrix cycles that run under the max reduction below
+    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
     alpha_prev = update_max(s_cur, sc);
     const float c = (kPShift - m_run) - kMagicF * sc;
     const uint8_t* kst = smem + ((j + 1) & (kStages - 1)) * kStageBytes;
@@ -257,8 +265,6 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         vf[i + 2 - 8] = v_frag(i + 2 - 8);
       s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i % 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
       const float e0 = p_of(s_cur[0][2 * i], sc, c), e1 = p_of(s_cur[0][2 * i + 1], sc, c);
-      l_part[(2 * i) & 3] += e0;
-      l_part[(2 * i + 1) & 3] += e1;
       if (i & 1) {
         int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, pf[i >> 1], true);
         pin(w);
@@ -275,18 +281,13 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt % 3], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
       float e[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        e[i] = p_of(s_cur[1][4 * dt + i], sc, c);
-        l_part[i] += e[i];
-      }
+      for (int i = 0; i < 4; ++i) e[i] = p_of(s_cur[1][4 * dt + i], sc, c);
       int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], 0, false);
       w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
       pin(w);
       pf[4 + dt] = w;
       __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) pin(l_part[i]);
     pf_prev = pf;
     // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
     tile_barrier();
@@ -306,6 +307,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const uint8_t* vst = smem + ((n_main - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_prev);
+    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
   }
   if (has_tail) {  // ragged last tile, not pipelined: mask keys >= Lk
     const int j = nkb - 1;
@@ -330,7 +332,6 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         for (int i = 0; i < 4; ++i) {
           const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
           e[i] = key < p.Lk ? p_of(s_cur[t][4 * g + i], sc, c) : 0.0f;
-          l_part[i] += e[i];
         }
         int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], 0, false);
         pf[4 * t + g] = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
@@ -338,12 +339,11 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const uint8_t* vst = smem + (j & (kStages - 1)) * kStageBytes + kTileBytes;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf);
+    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, lacc, 0, 0, 0, 0, 0, 0);
   }
 
   // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
-  const float l_lane = (l_part[0] + l_part[1]) + (l_part[2] + l_part[3]);
-  const float l_tot = l_lane + __shfl_xor(l_lane, 32);
-  const float inv_l = 1.0f / l_tot;
+  const float inv_l = 1.0f / lacc[0];
   const int q = q0 + l32;
   if (q < p.Lq) {
     uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;

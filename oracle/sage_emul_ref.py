@@ -7,7 +7,7 @@ v_scale):
 
     S  = (Q_i8 . K_i8^T) * q_scale * k_scale        integer dot products, exact
     P  = exp2(S - rowmax(S) + P_SHIFT)              Q already carries sm_scale * log2(e)
-    O  = (fp8(P) . V_fp8) * v_scale / rowsum(P)
+    O  = (fp8(P) . V_fp8) * v_scale / rowsum(fp8(P))
 
 It mirrors the kernel's tile-by-tile online softmax in fp32 (or, with ``online=False``, a
 full softmax), so it separates "error of the quantised
@@ -59,16 +59,16 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                     m_new = torch.maximum(m, st.amax(dim=1, keepdim=True))
                     alpha = torch.exp2(m - m_new)
                     p = torch.exp2(st - m_new + P_SHIFT)
-                    l = l * alpha + p.sum(dim=1, keepdim=True)
                     p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                    l = l * alpha + p8.sum(dim=1, keepdim=True)  # the normaliser sees the rounded P too
                     acc = acc * alpha + p8 @ vf[j0 : j0 + BLKK]
                     m = m_new
                 o = acc / l * v_scale[b, hk][None, :]
             else:
                 m = s.amax(dim=1, keepdim=True)
                 p = torch.exp2(s - m + P_SHIFT)
-                l = p.sum(dim=1, keepdim=True)
                 p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                l = p8.sum(dim=1, keepdim=True)
                 o = (p8 @ vf) * v_scale[b, hk][None, :] / l
             out[b, :, h, :] = o.to(out_dtype)
     return out
