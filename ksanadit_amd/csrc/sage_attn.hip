@@ -45,6 +45,20 @@ constexpr int kMaxKeyTiles = 4096;           // K scales of one head are kept in
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// 16 bytes per lane from global memory straight into LDS at `lds_dst + 16 * lane` (lds_dst is
+// wave-uniform).  Written as inline assembly on purpose: the compiler's wait-count model treats
+// the builtin form as a possible LDS access through the flat path and from then on waits for
+// ALL outstanding LDS reads before every use (lgkmcnt(0)), which serialises the operand
+// prefetch.  The copy is tracked by hand instead (vmcnt, see tile_barrier).
+// The global address is a wave-uniform base (scalar registers) plus a 32-bit per-lane offset.
+__device__ __forceinline__ void lds_copy16(const void* gbase, unsigned lane_off, const void* lds_dst) {
+  const unsigned lds_off = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)lds_dst;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_off), "v"(lane_off), "s"(gbase)
+               : "memory");
+}
+
 // Opaque use+def at this program point: keeps the optimizer from sinking the computation of
 // `x` into a later basic block (it emits no instruction).
 template <typename T>
@@ -132,12 +146,19 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   for (int r = 0; r < 16; ++r) lacc[r] = 0.0f;
   const v8i ones = {0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838};
 
+  // kept opaque so the 16 registers stay resident instead of being rebuilt from constants
+  // (8 moves) at every tile
   v16i magic;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) magic[r] = kMagicI;
+  for (int r = 0; r < 16; ++r) {
+    int m = kMagicI;
+    pin(m);
+    magic[r] = m;
+  }
 
-  const uint8_t* k_src = reinterpret_cast<const uint8_t*>(p.k_tiles) + (int64_t)bhk * p.nkb * kTileBytes + tid * 16;
-  const uint8_t* v_src = p.v_tiles + (int64_t)bhk * p.nkb * kTileBytes + tid * 16;
+  const uint8_t* k_src = reinterpret_cast<const uint8_t*>(p.k_tiles) + (int64_t)bhk * p.nkb * kTileBytes;  // uniform
+  const uint8_t* v_src = p.v_tiles + (int64_t)bhk * p.nkb * kTileBytes;
+  const unsigned copy_off = tid * 16;  // this lane's 16 bytes inside a tile
   const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb;
   const int nkb = p.nkb;
   // K scales live in LDS behind the ring: a per-tile global load would share the in-order
@@ -155,11 +176,9 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     // clamped: past the end the last tile is copied again into a stage nobody reads any more,
     // which keeps the loop free of branches and the outstanding-copy count constant
     const int jl = min(tile, nkb - 1);
-    uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes + wave * 1024;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(k_src + (int64_t)jl * kTileBytes),
-                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(v_src + (int64_t)jl * kTileBytes),
-                                     (__attribute__((address_space(3))) void*)(dst + kTileBytes), 16, 0, 0);
+    const uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes + wave * 1024;
+    lds_copy16(k_src + (int64_t)jl * kTileBytes, copy_off, dst);
+    lds_copy16(v_src + (int64_t)jl * kTileBytes, copy_off, dst + kTileBytes);
   };
   // wait until every copy except those of the newest (kAhead - 2) tiles has landed, then meet
   // the other waves.  Plain s_barrier: a fence here would drain ALL copies and undo the prefetch.
@@ -167,6 +186,10 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * (kAhead - 2)) : "memory");
   };
 
+  // Every ordinary global load above (Q fragments, scales) must have returned before the first
+  // asynchronous copy is issued: the compiler would otherwise drain ALL memory operations,
+  // copies included, at the first use of a loaded value inside the loop.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   // Stage 7's V half is read (times P = 0) by the first loop iteration: make it finite.
   *reinterpret_cast<uint4*>(smem + (kStages - 1) * kStageBytes + kTileBytes + tid * 16) = make_uint4(0, 0, 0, 0);
 #pragma unroll
@@ -190,13 +213,19 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
     lacc[0] *= alpha;
   };
-  // new running max of query l32 after the tile in s_cur; returns 2^(old max - new max)
-  auto update_max = [&](const v16i (&s_cur)[2], float sc) -> float {
-    int imax = s_cur[0][0];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) imax = max(imax, s_cur[t][r]);
+  // max over the 16 keys one S^T register block holds for query l32, as two independent chains
+  auto max8 = [&](const v16i& blk, int r0) {
+    int m = max(max(blk[r0], blk[r0 + 1]), blk[r0 + 2]);
+    m = max(max(m, blk[r0 + 3]), blk[r0 + 4]);
+    m = max(max(m, blk[r0 + 5]), blk[r0 + 6]);
+    return max(m, blk[r0 + 7]);
+  };
+  // this lane's maximum over a whole tile (32 of query l32's 64 keys)
+  auto lane_max = [&](const v16i (&blk)[2]) {
+    return max(max(max8(blk[0], 0), max8(blk[0], 8)), max(max8(blk[1], 0), max8(blk[1], 8)));
+  };
+  // new running max of query l32 given this lane's tile maximum; returns 2^(old max - new max)
+  auto update_max = [&](int imax, float sc) -> float {
     {
       // the other half of query l32's keys lives in lane l32 + 32
       int other = imax;
@@ -222,72 +251,85 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 
   v16i s_a[2], s_b[2];
   qk_tile(smem, lane, qf, magic, s_a);
+  int mx_cur = lane_max(s_a);  // this lane's maximum of the tile whose probabilities come next
+  float ks_cur = s_ks[0];
 
   // Software pipeline, one key tile per step.  While this tile's probabilities are computed on
   // the VALU, the matrix pipe runs the S^T MFMAs of the NEXT tile and the PV MFMAs of the
-  // PREVIOUS tile: every MFMA below is followed by the VALU work that hides it, and
-  // sched_barrier pins that order.  Because PV lags one tile, so does the rescaling of O:
+  // PREVIOUS tile: every MFMA below is followed by the VALU work that hides it, LDS operands are
+  // requested three MFMAs ahead, and sched_barrier pins that order.  The max reduction of the
+  // next tile rides in the PV chunks, so a step starts with only the short finalisation.
+  // Because PV lags one tile, so does the rescaling of O:
   //   at step j   O holds tiles <= j-2 relative to max m(j-2); alpha_prev = 2^(m(j-2) - m(j-1))
   //   step j      O *= alpha_prev (rare branch), then O += P(j-1) V(j-1), both relative to m(j-1)
   // LDS ring of 8 stages: tile j-1 (V), j (V next step), j+1 (K), j+2 .. j+4 (arriving).
   v8i pf_prev = {0, 0, 0, 0, 0, 0, 0, 0};
   float alpha_prev = 1.0f;
   auto tile_step = [&](int j, v16i (&s_cur)[2], v16i (&s_nxt)[2]) {
-    issue_copy(j + kAhead);
-    const float sc = qs * s_ks[j];
-    if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
-    // row sums of tile j-1: 64 matrix cycles that run under the max reduction below
-    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
-    alpha_prev = update_max(s_cur, sc);
-    const float c = (kPShift - m_run) - kMagicF * sc;
     const uint8_t* kst = smem + ((j + 1) & (kStages - 1)) * kStageBytes;
     const uint8_t* vst = smem + ((j - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
-    v8i pf;
-    // LDS operands are requested two MFMAs ahead of their use (12 fragments: 8 of K, 4 of V^T)
     auto k_frag = [&](int i) { return *reinterpret_cast<const v4i*>(kst + (((i & 1) * 4 + (i >> 1)) * 64 + lane) * 16); };
     auto v_frag = [&](int dt) {
       const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
       const v4i hi = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 1) * 64 + lane) * 16);
       return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
-    v4i kf[3];
-    v8i vf[3];
+    v4i kf[4];
+    v8i vf[4];
+    // operands of the first three S^T MFMAs and the next tile's K scale: requested before the
+    // dependent scalar work below, so their LDS latency is hidden behind it
     kf[0] = k_frag(0);
     kf[1] = k_frag(1);
+    kf[2] = k_frag(2);
+    const float ks_nxt = s_ks[min(j + 1, nkb - 1)];
+    issue_copy(j + kAhead);
+    if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
+    // row sums of tile j-1: 64 matrix cycles that run under the max finalisation below
+    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
+    const float sc = qs * ks_cur;
+    alpha_prev = update_max(mx_cur, sc);
+    const float c = (kPShift - m_run) - kMagicF * sc;
+    v8i pf;
+    int pm[4];
     __builtin_amdgcn_sched_barrier(0);
     // 8 x [S^T MFMA of tile j+1 (32 matrix cycles) | 2 probabilities of tile j]
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int s = i >> 1, t = i & 1;
-      if (i + 2 < 8)
-        kf[(i + 2) % 3] = k_frag(i + 2);
+      if (i + 3 < 8)
+        kf[(i + 3) & 3] = k_frag(i + 3);
       else
-        vf[i + 2 - 8] = v_frag(i + 2 - 8);
-      s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i % 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
+        vf[i + 3 - 8] = v_frag(i + 3 - 8);
+      s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i & 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
       const float e0 = p_of(s_cur[0][2 * i], sc, c), e1 = p_of(s_cur[0][2 * i + 1], sc, c);
       if (i & 1) {
         int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, pf[i >> 1], true);
         pin(w);
         pf[i >> 1] = w;
       } else {
-        pf[i >> 1] = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, 0, false);
+        pf[i >> 1] = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, __float_as_int(e0), false);  // both halves get written
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    // 4 x [PV MFMA of tile j-1 (64 matrix cycles) | 4 probabilities of tile j]
+    // 4 x [PV MFMA of tile j-1 (64 matrix cycles) | 4 probabilities of tile j | a quarter of
+    // the max reduction of tile j+1, whose S^T MFMAs were issued at least one chunk ago]
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
-      if (dt + 2 < 4) vf[(dt + 2) % 3] = v_frag(dt + 2);
-      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt % 3], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
+      if (dt == 0) vf[3] = v_frag(3);
+      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
       float e[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) e[i] = p_of(s_cur[1][4 * dt + i], sc, c);
-      int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], 0, false);
+      int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], __float_as_int(e[0]), false);
       w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
       pin(w);
       pf[4 + dt] = w;
+      pm[dt] = max8(s_nxt[dt >> 1], (dt & 1) * 8);
+      pin(pm[dt]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    mx_cur = max(max(pm[0], pm[1]), max(pm[2], pm[3]));
+    ks_cur = ks_nxt;
     pf_prev = pf;
     // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
     tile_barrier();
@@ -320,7 +362,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         if (key >= p.Lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
       }
     const float sc = qs * s_ks[j];
-    scale_o(update_max(s_cur, sc));
+    scale_o(update_max(lane_max(s_cur), sc));
     const float c = (kPShift - m_run) - kMagicF * sc;
     v8i pf;
 #pragma unroll
