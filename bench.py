@@ -30,6 +30,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default=None, help="one of ksanadit_amd.workloads.WORKLOADS (default: headline)")
+    ap.add_argument("--pwl-exp2", action="store_true", help="piecewise-linear e4m3 code instead of exp2 on the transcendental unit (faster, less accurate)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
     return ap.parse_args()
 
@@ -93,7 +94,7 @@ def main() -> int:
         sage_ops.quant_v(v, ws)
         if ev:
             ev[1].record()
-        sage_ops.attn_fwd(ws, out)
+        sage_ops.attn_fwd(ws, out, pwl_exp2=args.pwl_exp2)
         if ev:
             ev[2].record()
 
@@ -129,7 +130,8 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "int8+fp8",
         "data": "synthetic",
-        "config": {"workload": f"{w.name}: B={w.B} H={w.H} L={w.L} D={w.D} bf16 non-causal, seed {w.seed}"},
+        "config": {"workload": f"{w.name}: B={w.B} H={w.H} L={w.L} D={w.D} bf16 non-causal, seed {w.seed}",
+                   "exp2": "piecewise-linear e4m3 code" if args.pwl_exp2 else "exact"},
         "attn_kernel_ms": round(attn_ms, 4),
         "attn_kernel_tflops": round(attn_tflops, 2),
         "pct_mfma_peak": round(100.0 * attn_tflops / MFMA_PEAK_TFLOPS, 2),

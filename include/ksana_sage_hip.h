@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 1
+#define KSANA_SAGE_ABI_VERSION 2
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -41,6 +41,13 @@ extern "C" {
 #define KSANA_SAGE_EINVAL (-1)   /* bad shape, stride, alignment, dtype or null pointer      */
 #define KSANA_SAGE_ENOTSUP (-2)  /* valid request this build does not implement (D != 128, causal) */
 #define KSANA_SAGE_EHIP (-3)     /* the HIP runtime reported an error at launch               */
+
+/* flags of the attention entry points */
+#define KSANA_SAGE_FLAG_PWL_EXP2 1 /* Default (flag clear): P = exp2(x) on the transcendental unit, then the  */
+                                   /* hardware e4m3 cast.  Flag set: the e4m3 CODE of P is computed directly  */
+                                   /* as rne(8*x + 55.5), i.e. exp2 with a piecewise-linear 3-bit mantissa:   */
+                                   /* ~35 % fewer vector-ALU slots (about 1.2x faster), cos-sim to SDPA lower */
+                                   /* by ~1.5e-4 and the worst element about 2x further out.                  */
 
 /* rows per int8 scale: Q per token, K per 64 keys (sage_sla.py:190,204 uses (128, 64) off-Hopper;
  * the per-token Q scale is free in this kernel's operand layout and tighter) */
@@ -102,16 +109,16 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], con
 
 /* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
  * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel
- * call (sage_sla.py:237-253, dense form).  causal must be 0 in this build. */
+ * call (sage_sla.py:237-253, dense form).  causal must be 0 in this build; flags: KSANA_SAGE_FLAG_*. */
 int ksana_sage_attn_fwd(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
-                        const ksana_sage_shape* shape, int causal, void* stream);
+                        const ksana_sage_shape* shape, int causal, int flags, void* stream);
 
 /* The whole path in one call: quant_q, quant_k, quant_v, attn_fwd on `stream`.
  * Replaces sageattn(q, k, v, tensor_layout="NHD", is_causal=causal) (sage_attn.py:75-81). */
 int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype,
                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                        const int64_t o_strides[4], const ksana_sage_shape* shape, float sm_scale, int smooth_k,
-                       int causal, void* workspace, void* stream);
+                       int causal, int flags, void* workspace, void* stream);
 
 #ifdef __cplusplus
 }

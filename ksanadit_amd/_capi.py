@@ -11,10 +11,11 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
+FLAG_PWL_EXP2 = 1
 
 EXPORTS = (
     "ksana_sage_abi_version",
@@ -60,8 +61,8 @@ def _declare(lib):
     lib.ksana_sage_quant_q.argtypes, lib.ksana_sage_quant_q.restype = [vp, i, st, sp, f, vp, vp], i
     lib.ksana_sage_quant_k.argtypes, lib.ksana_sage_quant_k.restype = [vp, i, st, sp, i, vp, vp], i
     lib.ksana_sage_quant_v.argtypes, lib.ksana_sage_quant_v.restype = [vp, i, st, sp, vp, vp], i
-    lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, i, vp], i
-    lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, f, i, i, vp, vp]
+    lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, i, i, vp], i
+    lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward.restype = i
 
 

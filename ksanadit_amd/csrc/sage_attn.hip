@@ -98,7 +98,7 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
   }
 }
 
-template <int DT>
+template <int DT, bool kPwlExp>
 __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg, int n_wg,
                                                                      int wg_per_xcd) {
   // Consecutive workgroup ids land on consecutive XCDs (8 per chip, one L2 each).  Give every
@@ -241,6 +241,26 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   // p = exp2(sc*dot - m_run + shift); the magic is folded into the constant c, which is off by
   // at most ~1.5 integer steps of the dot product
   auto p_of = [&](int acc_bits, float sc, float c) { return fast_exp2(__builtin_fmaf(__int_as_float(acc_bits), sc, c)); };
+  // Four probabilities -> one dword of e4m3 codes (bytes in register order).
+  //   exact:  p = exp2(x) on the transcendental unit, then the hardware e4m3 conversion;
+  //   kPwlExp: the e4m3 CODE is computed directly, code = rne(8*x + 55.5) (saturating at 0): an
+  //           e4m3 code is a 3-bit-mantissa logarithm, so this is exp2 with a piecewise-linear
+  //           mantissa - two VALU slots per key instead of 3.5, no transcendental.  x <= 8 keeps
+  //           the code <= 120, clear of the NaN code 127.
+  auto pack4 = [&](int s0, int s1, int s2, int s3, float sc, float c) -> int {
+    if constexpr (kPwlExp) {
+      // here sc and c arrive pre-multiplied by 8, c with the +55.5 folded in
+      unsigned w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s0), sc, c), 0, 0u);
+      w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s1), sc, c), 1, w);
+      w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s2), sc, c), 2, w);
+      w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s3), sc, c), 3, w);
+      return (int)w;
+    } else {
+      const float e0 = p_of(s0, sc, c), e1 = p_of(s1, sc, c), e2 = p_of(s2, sc, c), e3 = p_of(s3, sc, c);
+      int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, __float_as_int(e0), false);  // both halves get written
+      return __builtin_amdgcn_cvt_pk_fp8_f32(e2, e3, w, true);
+    }
+  };
   // O^T += V^T . P^T for one 32-channel slice
   auto pv_slice = [&](const uint8_t* vst, int dt, const v8i& pf) {
     const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
@@ -288,7 +308,11 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
     const float sc = qs * ks_cur;
     alpha_prev = update_max(mx_cur, sc);
+    // exponent of key r: x = sc*dot - m_run + shift, with the magic folded into the constant
+    // (which is therefore off by at most ~1.5 integer steps of the dot product)
     const float c = (kPShift - m_run) - kMagicF * sc;
+    const float scp = kPwlExp ? 8.0f * sc : sc;
+    const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     v8i pf;
     int pm[4];
     __builtin_amdgcn_sched_barrier(0);
@@ -301,13 +325,22 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       else
         vf[i + 3 - 8] = v_frag(i + 3 - 8);
       s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i & 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
-      const float e0 = p_of(s_cur[0][2 * i], sc, c), e1 = p_of(s_cur[0][2 * i + 1], sc, c);
-      if (i & 1) {
-        int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, pf[i >> 1], true);
-        pin(w);
-        pf[i >> 1] = w;
+      if constexpr (kPwlExp) {
+        unsigned w = (i & 1) ? (unsigned)pf[i >> 1] : 0u;
+        w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s_cur[0][2 * i]), scp, cp), (2 * i) & 3, w);
+        w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s_cur[0][2 * i + 1]), scp, cp), (2 * i + 1) & 3, w);
+        int wi = (int)w;
+        if (i & 1) pin(wi);
+        pf[i >> 1] = wi;
       } else {
-        pf[i >> 1] = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, __float_as_int(e0), false);  // both halves get written
+        const float e0 = p_of(s_cur[0][2 * i], scp, cp), e1 = p_of(s_cur[0][2 * i + 1], scp, cp);
+        if (i & 1) {
+          int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, pf[i >> 1], true);
+          pin(w);
+          pf[i >> 1] = w;
+        } else {
+          pf[i >> 1] = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, __float_as_int(e0), false);  // both halves get written
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -317,11 +350,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     for (int dt = 0; dt < 4; ++dt) {
       if (dt == 0) vf[3] = v_frag(3);
       oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
-      float e[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) e[i] = p_of(s_cur[1][4 * dt + i], sc, c);
-      int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], __float_as_int(e[0]), false);
-      w = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
+      int w = pack4(s_cur[1][4 * dt], s_cur[1][4 * dt + 1], s_cur[1][4 * dt + 2], s_cur[1][4 * dt + 3], scp, cp);
       pin(w);
       pf[4 + dt] = w;
       pm[dt] = max8(s_nxt[dt >> 1], (dt & 1) * 8);
@@ -364,19 +393,22 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const float sc = qs * s_ks[j];
     scale_o(update_max(lane_max(s_cur), sc));
     const float c = (kPShift - m_run) - kMagicF * sc;
+    const float scp = kPwlExp ? 8.0f * sc : sc;
+    const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     v8i pf;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float e[4];
+        const int w = pack4(s_cur[t][4 * g], s_cur[t][4 * g + 1], s_cur[t][4 * g + 2], s_cur[t][4 * g + 3], scp, cp);
+        // zero the bytes of keys at or beyond Lk (code 0 is +0.0 in e4m3)
+        unsigned keep = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
-          e[i] = key < p.Lk ? p_of(s_cur[t][4 * g + i], sc, c) : 0.0f;
+          if (key < p.Lk) keep |= 0xffu << (8 * i);
         }
-        int w = __builtin_amdgcn_cvt_pk_fp8_f32(e[0], e[1], 0, false);
-        pf[4 * t + g] = __builtin_amdgcn_cvt_pk_fp8_f32(e[2], e[3], w, true);
+        pf[4 * t + g] = w & (int)keep;
       }
     const uint8_t* vst = smem + (j & (kStages - 1)) * kStageBytes + kTileBytes;
 #pragma unroll
@@ -403,6 +435,18 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   }
 }
 
+template <int DT, bool kPwlExp>
+hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
+                          hipStream_t s) {
+  // more than 64 KiB of dynamic LDS has to be requested per kernel, once per process
+  static const hipError_t attr =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStageBytes + kMaxKeyTiles * 4);
+  if (attr != hipSuccess) return attr;
+  sage_attn_fwd_kernel<DT, kPwlExp><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
@@ -413,20 +457,12 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const dim3 grid(wg_per_xcd * 8), block(kThreadsAttn);
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
   const size_t lds = kStages * kStageBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
-  // more than 64 KiB of dynamic LDS has to be requested per kernel, once
-  static const hipError_t attr_bf16 = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&sage_attn_fwd_kernel<KSANA_SAGE_BF16>), hipFuncAttributeMaxDynamicSharedMemorySize,
-      kStages * kStageBytes + kMaxKeyTiles * 4);
-  static const hipError_t attr_fp16 = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&sage_attn_fwd_kernel<KSANA_SAGE_FP16>), hipFuncAttributeMaxDynamicSharedMemorySize,
-      kStages * kStageBytes + kMaxKeyTiles * 4);
-  if (attr_bf16 != hipSuccess) return attr_bf16;
-  if (attr_fp16 != hipSuccess) return attr_fp16;
-  if (p.o.dtype == KSANA_SAGE_BF16)
-    sage_attn_fwd_kernel<KSANA_SAGE_BF16><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
-  else
-    sage_attn_fwd_kernel<KSANA_SAGE_FP16><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
-  return hipGetLastError();
+  const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
+  if (p.exact_exp2)
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
+  return bf16 ? launch_variant<KSANA_SAGE_BF16, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
+              : launch_variant<KSANA_SAGE_FP16, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
 }
 
 }  // namespace ksana_sage

@@ -173,9 +173,10 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksan
 }
 
 int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
-                        int causal, void* stream) {
+                        int causal, int flags, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
+  if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
   ksana_sage_ws_layout l;
@@ -190,13 +191,15 @@ int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4
   p.o = ksana_sage::OutTensor{static_cast<uint16_t*>(o), o_st[0], o_st[1], o_st[2], dtype};
   p.B = s->B, p.Hq = s->Hq, p.Hkv = s->Hkv, p.Lq = s->Lq, p.Lk = s->Lk;
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;
+  p.exact_exp2 = (flags & KSANA_SAGE_FLAG_PWL_EXP2) ? 0 : 1;
   hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
 }
 
 int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
                        const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
-                       const ksana_sage_shape* s, float sm_scale, int smooth_k, int causal, void* ws, void* stream) {
+                       const ksana_sage_shape* s, float sm_scale, int smooth_k, int causal, int flags, void* ws,
+                       void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
   // validate everything before the first launch so a bad argument leaves no partial work
@@ -208,7 +211,7 @@ int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int
   if (int rc = ksana_sage_quant_q(q, dtype, q_st, s, sm_scale, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_k(k, dtype, k_st, s, smooth_k, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_v(v, dtype, v_st, s, ws, stream)) return rc;
-  return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, causal, stream);
+  return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, causal, flags, stream);
 }
 
 }  // extern "C"

@@ -49,6 +49,7 @@ struct AttnParams {
   const float* v_scale;
   OutTensor o;
   int B, Hq, Hkv, Lq, Lk, lq_pad, nkb;
+  int exact_exp2;  // 1: exp2 on the transcendental unit; 0: piecewise-linear e4m3 code (faster)
 };
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s);
 

@@ -145,11 +145,12 @@ def quant_v(v: torch.Tensor, ws: SageWorkspace) -> None:
     _capi.check(rc, "ksana_sage_quant_v")
 
 
-def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False) -> torch.Tensor:
+def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False) -> torch.Tensor:
     _require_hip(out)
     lib = _capi.load()
+    flags = _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0
     rc = lib.ksana_sage_attn_fwd(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
-                                 int(causal), _stream_ptr(out.device))
+                                 int(causal), flags, _stream_ptr(out.device))
     _capi.check(rc, "ksana_sage_attn_fwd")
     return out
 
@@ -163,8 +164,12 @@ def sageattn(
     sm_scale: float | None = None,
     smooth_k: bool = True,
     workspace: SageWorkspace | None = None,
+    pwl_exp2: bool = False,
 ) -> torch.Tensor:
-    """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out."""
+    """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
+
+    ``pwl_exp2=True`` computes the e4m3 code of every probability directly (exp2 with a
+    piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate."""
     if tensor_layout not in ("NHD", "HND"):
         raise ValueError(f"tensor_layout {tensor_layout!r} unknown")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -183,7 +188,7 @@ def sageattn(
     rc = lib.ksana_sage_forward(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
         _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape),
-        sm_scale, int(smooth_k), int(is_causal), ws.ptr, _stream_ptr(q.device),
+        sm_scale, int(smooth_k), int(is_causal), _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
     )
     _capi.check(rc, "ksana_sage_forward")
     return out.transpose(1, 2) if tensor_layout == "HND" else out

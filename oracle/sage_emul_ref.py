@@ -6,7 +6,8 @@ the kernel signature visible at sage_sla.py:237-253 (q_int8, k_int8, v_fp8, q_sc
 v_scale):
 
     S  = (Q_i8 . K_i8^T) * q_scale * k_scale        integer dot products, exact
-    P  = exp2(S - rowmax(S) + P_SHIFT)              Q already carries sm_scale * log2(e)
+    P  = exp2(S - rowmax(S) + P_SHIFT)              Q already carries sm_scale * log2(e); exp2 either
+                                                    exact or with a piecewise-linear mantissa (p_to_e4m3)
     O  = (fp8(P) . V_fp8) * v_scale / rowsum(fp8(P))
 
 It mirrors the kernel's tile-by-tile online softmax in fp32 (or, with ``online=False``, a
@@ -20,14 +21,28 @@ from __future__ import annotations
 
 import torch
 
-from .quant_ref import BLKK, BLKQ, FP8_MAX, quant_k_ref, quant_q_ref, quant_v_ref
+from .quant_ref import BLKK, BLKQ, FP8_MAX, e4m3fn_decode_table, quant_k_ref, quant_q_ref, quant_v_ref
 
 # P is scaled by 2**P_SHIFT before the fp8 cast so that small probabilities stay above the
 # e4m3 subnormal floor (2**-9); the factor cancels in O = (P V) / rowsum(P).
 P_SHIFT = 8.0
 
 
-def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True):
+def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
+    """x = log2 of the (shifted) probability -> the e4m3 value the kernel feeds to the PV MFMA.
+
+    exact (default): round(exp2(x)) to e4m3 (nearest even).
+    otherwise: the e4m3 CODE is rne(8*x + 55.5) clamped to [0, 126]; decoding it gives
+    2^floor(.) * (1 + m/8): exp2 with a piecewise-linear 3-bit mantissa (codes below 8 are the
+    subnormals, so probabilities under 2^-14 of the row maximum fade to zero linearly)."""
+    if exact_exp2:
+        return torch.exp2(x).clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+    code = torch.round(8.0 * x + 55.5).clamp_(0, 126).long()
+    return e4m3fn_decode_table().float()[code]
+
+
+def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True,
+                         exact_exp2=True):
     """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
 
     ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
@@ -51,34 +66,53 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 s = s.masked_fill(~mask, float("-inf"))
             vf = v_fp8[b, hk].float()
             if online:
+                # Mirrors the kernel's arithmetic operation by operation (fp32, FMAs emulated in
+                # float64) so that e4m3 codes agree except at exact rounding ties:
+                #   x_f = float(MAGIC + dot)            the int32 accumulator read as fp32
+                #   sc  = q_scale * k_scale             one fp32 product per (row, tile)
+                #   c   = (SHIFT - m) - MAGIC * sc      fp32, in this order
+                #   exponent = fma(x_f, sc, c)          (pwl: fma(x_f, 8 sc, fma(8, c, 55.5)))
+                magic = 12582912.0
+                x_f = (s_int + magic).to(torch.float32)  # exact: |dot| < 2**22
                 m = torch.full((Lq, 1), float("-inf"))
                 l = torch.zeros(Lq, 1)
                 acc = torch.zeros(Lq, D)
+                if causal:
+                    raise NotImplementedError("online emulation of causal masking")
                 for j0 in range(0, Lk, BLKK):
-                    st = s[:, j0 : j0 + BLKK]
-                    m_new = torch.maximum(m, st.amax(dim=1, keepdim=True))
+                    sc = (qs_row[b, h][:, None] * k_scale[b, hk, j0 // BLKK]).to(torch.float32)
+                    xt = x_f[:, j0 : j0 + BLKK]
+                    m_tile = (xt.amax(dim=1, keepdim=True) - magic) * sc
+                    m_new = torch.maximum(m, m_tile)
                     alpha = torch.exp2(m - m_new)
-                    p = torch.exp2(st - m_new + P_SHIFT)
-                    p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                    c = (P_SHIFT - m_new) - magic * sc
+                    if exact_exp2:
+                        e = (xt.double() * sc.double() + c.double()).float()
+                        p8 = torch.exp2(e).clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                    else:
+                        cp = (8.0 * c.double() + 55.5).float()
+                        t = (xt.double() * (8.0 * sc).double() + cp.double()).float()
+                        code = torch.round(t).clamp_(0, 126).long()
+                        p8 = e4m3fn_decode_table().float()[code]
                     l = l * alpha + p8.sum(dim=1, keepdim=True)  # the normaliser sees the rounded P too
                     acc = acc * alpha + p8 @ vf[j0 : j0 + BLKK]
                     m = m_new
                 o = acc / l * v_scale[b, hk][None, :]
             else:
                 m = s.amax(dim=1, keepdim=True)
-                p = torch.exp2(s - m + P_SHIFT)
-                p8 = p.clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
+                p8 = p_to_e4m3(s - m + P_SHIFT, exact_exp2)
                 l = p8.sum(dim=1, keepdim=True)
                 o = (p8 @ vf) * v_scale[b, hk][None, :] / l
             out[b, :, h, :] = o.to(out_dtype)
     return out
 
 
-def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True):
+def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True, exact_exp2=True):
     """[B, L, H, D] half in, same out: quantise with the oracle quantizer, then emulate."""
     D = q.shape[-1]
     sm_scale = D**-0.5 if sm_scale is None else sm_scale
     q_i8, q_scale = quant_q_ref(q, sm_scale)
     k_i8, k_scale, _ = quant_k_ref(k, smooth_k=smooth_k)
     v_fp8, v_scale = quant_v_ref(v)
-    return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal, online=online)
+    return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal, online=online,
+                                exact_exp2=exact_exp2)

@@ -29,11 +29,11 @@ def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
     return q.to(dtype), k.to(dtype), v.to(dtype)
 
 
-def _emul_from_ws(ws, Lq, Lk, dtype):
+def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True):
     """The CPU emulation fed with the operands the GPU quantizer actually produced."""
     return sage_emul_from_quant(
         ws.q_i8.cpu()[:, :, :Lq], ws.q_scale.cpu()[:, :, :Lq], untile_k(ws.k_tiles.cpu(), Lk), ws.k_scale.cpu(),
-        untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), dtype,
+        untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), dtype, exact_exp2=exact_exp2,
     )
 
 
@@ -42,20 +42,21 @@ def _emul_from_ws(ws, Lq, Lk, dtype):
     [(1, 64, 64, 1, 1), (1, 256, 256, 2, 2), (2, 300, 300, 3, 3), (1, 32, 1, 1, 1), (1, 1, 70, 2, 2),
      (1, 257, 65, 2, 1), (1, 700, 512, 4, 4), (1, 100, 1000, 2, 2)],
 )
-def test_attention_vs_oracles_small(hip_device, B, Lq, Lk, Hq, Hkv):
-    print(f"case B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv}", flush=True)
+@pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
+def test_attention_vs_oracles_small(hip_device, B, Lq, Lk, Hq, Hkv, exact):
+    print(f"case B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv} exact_exp2={exact}", flush=True)
     q, k, v = _rand_qkv(B, Lq, Lk, Hq, Hkv, seed=Lq + 3 * Lk)
     qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
     ws = sage_ops.workspace_for(qd, kd)
     ws.blob.fill_(0x7F)
-    out = sage_ops.sageattn(qd, kd, vd, workspace=ws)
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, pwl_exp2=not exact)
     torch.cuda.synchronize()
     assert out.shape == q.shape and out.dtype == q.dtype and out.is_contiguous()
     out = out.cpu()
     assert torch.isfinite(out.float()).all()
     # 1. kernel vs the emulation on the SAME quantized operands: only summation order, the online
     #    rescaling and the final bf16 rounding differ -> tight
-    emul = _emul_from_ws(ws, Lq, Lk, q.dtype)
+    emul = _emul_from_ws(ws, Lq, Lk, q.dtype, exact)
     scale = max(emul.float().abs().max().item(), 1e-3)
     diff = (out.float() - emul.float()).abs()
     # an exp2 that lands within an ulp of an e4m3 rounding boundary may round the other way
@@ -67,7 +68,8 @@ def test_attention_vs_oracles_small(hip_device, B, Lq, Lk, Hq, Hkv):
     #    absolute bound scales with the output magnitude here (2e-2 absolute holds from L=1560 on).
     ref = sdpa_ref(q, k, v)
     if Lk >= 64:
-        assert _cos(out, ref) >= COS_MIN
+        # the piecewise-linear exp2 sits ~1.5e-4 lower; on a handful of rows that can dip under the bar
+        assert _cos(out, ref) >= (COS_MIN if exact else 0.9985)
     assert (out.float() - ref.float()).abs().max() <= 0.12 * max(ref.float().abs().max().item(), 0.1)
 
 
@@ -129,18 +131,19 @@ def test_k_offset_invariance_and_determinism(hip_device):
     assert _cos(rough.cpu(), ref) < _cos(a.cpu(), ref)
 
 
+@pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
 @pytest.mark.parametrize("name,heads", [("cpu_plumbing", None), ("qwen_cfg", 6), ("wan14b_480p", 1)])
-def test_workloads_vs_cpu_sdpa_oracle(hip_device, name, heads):
-    print(f"workload {name} heads={heads}", flush=True)
+def test_workloads_vs_cpu_sdpa_oracle(hip_device, name, heads, exact):
+    print(f"workload {name} heads={heads} exact_exp2={exact}", flush=True)
     q, k, v = make_inputs(name, heads=heads)
     ref = sdpa_ref(q, k, v)
-    out = sage_ops.sageattn(*(t.to(hip_device) for t in (q, k, v))).cpu()
+    out = sage_ops.sageattn(*(t.to(hip_device) for t in (q, k, v)), pwl_exp2=not exact).cpu()
     c = _cos(out, ref)
     err = (out.float() - ref.float()).abs()
     print(f"{name}: cos={c:.6f} max_abs={err.max().item():.4e} mean_abs={err.mean().item():.4e} ref_max={ref.float().abs().max().item():.3f}", flush=True)
     assert c >= COS_MIN
     if name == "cpu_plumbing":
-        assert err.max().item() <= MAX_ABS_FLAT
+        assert err.max().item() <= (MAX_ABS_FLAT if exact else 2 * MAX_ABS_FLAT)
     else:
         # peaked attention (outlier / text tokens): |O| ~ |V| ~ 1-5, so a max-abs bound has to be
         # relative: two e4m3 roundings (2 x 2^-4) plus int8 logit noise on near-tied top keys

@@ -337,9 +337,14 @@ def test_sage_emul_meets_stated_tolerance_on_plumbing_workload():
     from ksanadit_amd.workloads import make_inputs
 
     q, k, v = make_inputs("cpu_plumbing", heads=2)
-    ref, out = sdpa_ref(q, k, v), sage_emul_ref(q, k, v)
+    ref = sdpa_ref(q, k, v)
+    out = sage_emul_ref(q, k, v)
     assert _cos(out, ref) >= 0.999
     assert (out.float() - ref.float()).abs().max() <= 2e-2
+    # the piecewise-linear exp2 keeps the cosine bar; its worst element is ~2x further out
+    fast = sage_emul_ref(q, k, v, exact_exp2=False)
+    assert _cos(fast, ref) >= 0.999
+    assert (fast.float() - ref.float()).abs().max() <= 4e-2
 
 
 def test_sage_emul_survives_outliers():
