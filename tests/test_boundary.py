@@ -1,0 +1,203 @@
+"""Host-side contract of the attention op and the C ABI; runs without a GPU.
+
+Mirrors the reference's own boundary behaviour: selector errors (backends/base.py:54-73), the op's
+argument checks (attention_op.py:41-42, 80-81), config validation (attention_config.py:79-83),
+shape/no-NaN checks of tests/ksana/attention_op_test.py:59-79, and the library's argument validation.
+"""
+
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+import ksanadit_amd
+from ksanadit_amd import KsanaAttentionBackend, KsanaAttentionConfig, KsanaAttentionOp, _capi, pick_attn_op, sage_ops
+from ksanadit_amd.backends import get_attention_backend_impl, get_backend_mapping
+from ksanadit_amd.backends.sage_attn import SageAttentionImpl
+from ksanadit_amd.backends.sdpa import SDPAImpl
+from ksanadit_amd.layout import TILE_BYTES, k_tile_index, v_tile_index
+from ksanadit_amd.workloads import HEADLINE, WORKLOADS, make_inputs
+from oracle.sdpa_ref import sdpa_ref
+
+ROOT = Path(__file__).resolve().parent.parent
+HAS_GPU = torch.cuda.is_available()
+
+
+# ----------------------------------------------------------------------------- C ABI
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "ksana_sage_hip.h").read_text()
+    declared = set(re.findall(r"\b(ksana_sage_[a-z_0-9]+)\s*\(", header))
+    assert declared >= {"ksana_sage_forward", "ksana_sage_attn_fwd", "ksana_sage_quant_q", "ksana_sage_quant_k",
+                        "ksana_sage_quant_v", "ksana_sage_workspace_layout", "ksana_sage_last_error", "ksana_sage_abi_version"}
+    lib = C.CDLL(str(_capi.LIB_PATH))
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert set(_capi.EXPORTS) == declared
+    version = int(re.search(r"#define KSANA_SAGE_ABI_VERSION (\d+)", header).group(1))
+    assert _capi.load().ksana_sage_abi_version() == version == _capi.ABI_VERSION
+
+
+def test_workspace_layout_headline_shape():
+    w = WORKLOADS[HEADLINE]
+    shape, lay = _capi.workspace_layout(w.B, w.H, w.H, w.L, w.L, w.D)
+    assert (lay.lq_pad, lay.nkb, lay.nch) == (32768, 512, 128)
+    offs = [lay.q_i8, lay.q_scale, lay.k_i8, lay.k_scale, lay.k_mean, lay.v_fp8, lay.v_scale, lay.v_inv, lay.k_part, lay.v_part]
+    assert offs == sorted(offs) and all(o % 256 == 0 for o in offs) and lay.total_bytes % 256 == 0
+    assert lay.q_scale - lay.q_i8 == w.H * 32768 * 128  # int8 Q, padded to 128 rows
+    assert lay.k_scale - lay.k_i8 == w.H * 512 * TILE_BYTES
+    assert lay.total_bytes < 3 * w.elements + (16 << 20)  # three 8-bit tensors, scales, partial sums
+
+
+@pytest.mark.parametrize(
+    "args,exc",
+    [((1, 4, 4, 16, 16, 64), NotImplementedError), ((1, 4, 3, 16, 16, 128), ValueError), ((1, 4, 4, 0, 16, 128), ValueError),
+     ((0, 4, 4, 16, 16, 128), ValueError), ((1, 4, 4, 16, 262145, 128), NotImplementedError), ((1, 70000, 70000, 16, 16, 128), ValueError)],
+)
+def test_workspace_layout_rejects_bad_shapes(args, exc):
+    with pytest.raises(exc):
+        _capi.workspace_layout(*args)
+
+
+def test_entry_points_validate_before_touching_the_gpu():
+    lib = _capi.load()
+    shape = _capi.Shape(1, 2, 2, 64, 64, 128)
+    st = _capi.Strides(64 * 2 * 128, 2 * 128, 128, 1)
+    null = C.c_void_p(0)
+    fake = C.c_void_p(0x1000)  # aligned, never dereferenced: every call below fails validation first
+    assert lib.ksana_sage_workspace_layout(None, None) == _capi.EINVAL
+    assert lib.ksana_sage_quant_q(null, _capi.BF16, st, C.byref(shape), 0.1, fake, null) == _capi.EINVAL
+    assert b"q is null" in lib.ksana_sage_last_error()
+    assert lib.ksana_sage_quant_k(fake, 7, st, C.byref(shape), 1, fake, null) == _capi.EINVAL  # dtype
+    assert lib.ksana_sage_quant_v(C.c_void_p(0x1008), _capi.BF16, st, C.byref(shape), fake, null) == _capi.EINVAL  # alignment
+    bad = _capi.Strides(64 * 2 * 128, 2 * 128, 128, 2)
+    assert lib.ksana_sage_quant_q(fake, _capi.BF16, bad, C.byref(shape), 0.1, fake, null) == _capi.EINVAL
+    assert b"D stride" in lib.ksana_sage_last_error()
+    odd = _capi.Strides(64 * 2 * 128, 2 * 128 + 4, 128, 1)
+    assert lib.ksana_sage_quant_q(fake, _capi.BF16, odd, C.byref(shape), 0.1, fake, null) == _capi.EINVAL
+    assert lib.ksana_sage_quant_q(fake, _capi.BF16, st, C.byref(shape), 0.1, null, null) == _capi.EINVAL  # workspace
+    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), 1, 0, null) == _capi.ENOTSUP  # causal
+    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), 0, 0x10, null) == _capi.EINVAL  # flags
+    assert lib.ksana_sage_forward(fake, fake, null, fake, _capi.BF16, st, st, st, st, C.byref(shape), 0.1, 1, 0, 0, fake, null) == _capi.EINVAL
+    with pytest.raises(ValueError):
+        _capi.check(_capi.EINVAL, "x")
+    with pytest.raises(NotImplementedError):
+        _capi.check(_capi.ENOTSUP, "x")
+    with pytest.raises(_capi.SageLibraryError):
+        _capi.check(_capi.EHIP, "x")
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    monkeypatch.setattr(_capi, "_lib", None)
+    monkeypatch.setattr(_capi, "LIB_PATH", tmp_path / "libksana_sage_hip.so")
+    with pytest.raises(_capi.SageLibraryError, match="ksanadit_amd.build"):
+        _capi.load()
+    (tmp_path / "libksana_sage_hip.so").write_bytes(b"not an ELF file")
+    with pytest.raises(_capi.SageLibraryError, match="cannot load"):
+        _capi.load()
+
+
+def test_tile_index_maps_are_permutations():
+    for idx in (k_tile_index(), v_tile_index()):
+        assert idx.shape == (64, 128)
+        assert torch.equal(idx.flatten().sort().values, torch.arange(TILE_BYTES))
+    # a K operand fragment is 16 consecutive channels of one key; a V^T fragment is 4 consecutive keys
+    assert (k_tile_index()[5, 16:32] - k_tile_index()[5, 16] == torch.arange(16)).all()
+    assert (v_tile_index()[8:12, 7] - v_tile_index()[8, 7] == torch.arange(4)).all()
+
+
+# ----------------------------------------------------------------------------- selector / op
+def test_enum_values_and_supported_list_follow_the_reference():
+    assert KsanaAttentionBackend.SAGE_ATTN.value == "sage_attention" and KsanaAttentionBackend.TORCH_SDPA.value == "torch_sdpa"
+    assert KsanaAttentionBackend.get_supported_list() == ["sage_attention", "torch_sdpa"]
+    assert KsanaAttentionBackend.get_supported_list(exclude=[KsanaAttentionBackend.SAGE_ATTN]) == ["torch_sdpa"]
+    assert KsanaAttentionBackend.support("torch_sdpa") and not KsanaAttentionBackend.support("flash_attention")
+    assert KsanaAttentionBackend.support(KsanaAttentionBackend.FLASH_ATTN) and not KsanaAttentionBackend.support(3)
+    mapping = get_backend_mapping()
+    assert mapping[KsanaAttentionBackend.SAGE_ATTN] is SageAttentionImpl and mapping[KsanaAttentionBackend.TORCH_SDPA] is SDPAImpl
+
+
+def test_config_and_selector_errors():
+    with pytest.raises(ValueError):  # attention_config.py:79-83
+        KsanaAttentionConfig(backend="no_such_backend")
+    with pytest.raises(ValueError):
+        KsanaAttentionConfig(backend="flash_attention")  # known to the reference, not built here
+    with pytest.raises(ValueError):  # attention_op.py:41-42
+        KsanaAttentionOp(4, 128)
+    cfg = KsanaAttentionConfig(backend=KsanaAttentionBackend.FLASH_ATTN)  # enum members pass the config check ...
+    with pytest.raises(ValueError):  # ... and fail in the registry (base.py:62-63)
+        get_attention_backend_impl(cfg, head_size=128, dtype=torch.bfloat16)
+    frozen = KsanaAttentionConfig(backend="torch_sdpa")
+    with pytest.raises(Exception):
+        frozen.backend = "sage_attention"
+
+
+def test_no_backend_available_raises_runtime_error(monkeypatch):
+    monkeypatch.setattr(SageAttentionImpl, "supports", staticmethod(lambda **_: False))
+    monkeypatch.setattr(SDPAImpl, "supports", staticmethod(lambda **_: False))
+    with pytest.raises(RuntimeError, match="No compatible attention"):
+        get_attention_backend_impl(KsanaAttentionConfig(backend="torch_sdpa"), head_size=128, dtype=torch.float16)
+
+
+@pytest.mark.skipif(HAS_GPU, reason="describes the GPU-less host")
+def test_sage_request_on_a_host_without_gpu():
+    """supports() is False, the walk moves on to SDPA, and constructing SDPA under a Sage config
+    trips check_config - exactly what the reference does without its package (base.py:59-69,102-106)."""
+    assert SageAttentionImpl.supports(head_size=128, dtype=torch.bfloat16) is False
+    cfg = KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN)
+    assert get_attention_backend_impl(cfg, head_size=128, dtype=torch.bfloat16) is SDPAImpl
+    op = pick_attn_op(cfg)(num_heads=2, head_size=128)
+    q = torch.zeros(1, 8, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="does not match implementation"):
+        op(q, q, q)
+    with pytest.raises(RuntimeError):
+        SageAttentionImpl(cfg, 2, 128, False, 128**-0.5)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        sage_ops.sageattn(q, q, q)
+
+
+def test_sdpa_backend_on_cpu_matches_oracle_and_reference_checks():
+    B, L, H, D = 2, 32, 64, 128  # the reference's test shape, attention_op_test.py:24
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(B, L, H, D, dtype=torch.float16) for _ in range(3))
+    attn = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.TORCH_SDPA))(num_heads=H, head_size=D, causal=False)
+    assert attn.backend_type is None
+    out = attn(q, k, v, k_lens=None, window_size=(-1, -1), block_id=3, dense_only=True)  # model kwargs are tolerated
+    assert attn.backend_type == KsanaAttentionBackend.TORCH_SDPA
+    assert out.shape == q.shape and not torch.isnan(out).any()
+    assert torch.equal(out, sdpa_ref(q, k, v))
+    assert attn.softmax_scale == D**-0.5
+    # dtype change rebuilds the impl (attention_op.py:53-55); fp32 works on SDPA
+    first = attn._attn_impl
+    out32 = attn(q.float(), k.float(), v.float())
+    assert out32.dtype == torch.float32 and attn._attn_impl is not first
+    # per-call scale override and GQA (sdpa.py:52-75)
+    kk, vv = k[:, :, :8], v[:, :, :8]
+    assert torch.equal(attn(q, kk, vv, softmax_scale=0.2), sdpa_ref(q, kk, vv, scale=0.2))
+    for bad in (q[0], q.unsqueeze(0)):
+        with pytest.raises(ValueError, match=r"\[B, L, H, D\]"):
+            attn(bad, k, v)
+
+
+def test_cpu_plumbing_workload_through_the_op():
+    """configs[0]: the CPU-runnable case goes through this package's SDPA backend."""
+    q, k, v = make_inputs("cpu_plumbing", heads=2)
+    assert q.shape == (1, 1560, 2, 128) and q.dtype == torch.bfloat16
+    attn = pick_attn_op(KsanaAttentionConfig(backend="torch_sdpa"))(num_heads=2, head_size=128)
+    out = attn(q, k, v)
+    assert out.shape == q.shape and torch.isfinite(out.float()).all()
+    assert torch.equal(out, sdpa_ref(q, k, v))
+
+
+def test_workload_table():
+    w = WORKLOADS[HEADLINE]
+    assert (w.B, w.H, w.L, w.D) == (1, 40, 32760, 128) and abs(w.flops - 21.98e12) < 0.01e12
+    assert [WORKLOADS[n].L for n in ("cpu_plumbing", "wan5b_720p", "wan14b_720p", "qwen_cfg")] == [1560, 27280, 75600, 4352]
+    q1, k1, _ = make_inputs("qwen_cfg", heads=1, seq=600)
+    q2, k2, _ = make_inputs("qwen_cfg", heads=1, seq=600)
+    assert torch.equal(q1, q2) and torch.equal(k1, k2)  # seeded
+    assert q1[:, :256].float().std() > 2.0 * q1[:, 256:].float().std()  # text tokens first, N(0, 3)
+    qo, ko, _ = make_inputs("wan14b_480p", heads=1, seq=4096)
+    assert qo.float().abs().max() > 20 and ko.float().abs().max() > 20  # x20 outliers present
+    assert ksanadit_amd.DEFAULT_ATTENTION_BACKEND == KsanaAttentionBackend.SAGE_ATTN
