@@ -99,26 +99,58 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
   }
 }
 
-// chunk sums -> mean rounded to the input dtype, stored widened.  grid = B*H, 128 threads.
-__global__ __launch_bounds__(kD) void k_mean_finalize_kernel(const float* __restrict__ part, int nch, int L, int dtype,
-                                                             int smooth, float* __restrict__ k_mean) {
-  const int bh = blockIdx.x, d = threadIdx.x;
-  const float* p = part + (int64_t)bh * nch * kD + d;
-  float tot = nch > 0 ? p[0] : 0.0f;
-  for (int c = 1; c < nch; ++c) tot = tot + p[(int64_t)c * kD];
-  const float mean = __fdiv_rn(tot, (float)L);
-  k_mean[bh * kD + d] = smooth ? round_to_half_dtype(mean, dtype) : 0.0f;
+// Finalisation of the column reductions.  grid = B*H, 1024 threads.  All chunk partials of the
+// head are first pulled into LDS with independent, coalesced loads (the naive form - one
+// dependent global load per chunk - costs a memory latency per chunk); 128 threads then combine
+// them in increasing chunk order, which for the sum is part of the specification.
+constexpr int kFinThreads = 1024;
+constexpr int kFinMaxChunks = 96;  // partials staged per pass: 96 x 128 floats = 48 KiB of LDS
+
+template <int OP>
+__device__ __forceinline__ float combine_partials(const float* __restrict__ part, int nch, float* s_part) {
+  const int d = threadIdx.x & (kD - 1), sub = threadIdx.x >> 7;  // 8 loader groups
+  float acc = 0.0f;
+  bool first = true;
+  for (int c0 = 0; c0 < nch; c0 += kFinMaxChunks) {
+    const int n = min(kFinMaxChunks, nch - c0);
+    __syncthreads();
+    for (int c = sub; c < n; c += kFinThreads / kD) s_part[c * kD + d] = part[(int64_t)(c0 + c) * kD + d];
+    __syncthreads();
+    if (threadIdx.x < kD) {
+      for (int c = 0; c < n; ++c) {
+        const float v = s_part[c * kD + d];
+        acc = first ? v : (OP == 0 ? acc + v : fmaxf(acc, v));
+        first = false;
+      }
+    }
+  }
+  return acc;
 }
 
-__global__ __launch_bounds__(kD) void v_scale_finalize_kernel(const float* __restrict__ part, int nch,
-                                                              float* __restrict__ v_scale, float* __restrict__ v_inv) {
-  const int bh = blockIdx.x, d = threadIdx.x;
-  const float* p = part + (int64_t)bh * nch * kD + d;
-  float amax = p[0];
-  for (int c = 1; c < nch; ++c) amax = fmaxf(amax, p[(int64_t)c * kD]);
-  const bool nz = amax > 0.0f;
-  v_scale[bh * kD + d] = nz ? __fdiv_rn(amax, 448.0f) : 0.0f;
-  v_inv[bh * kD + d] = nz ? __fdiv_rn(448.0f, amax) : 0.0f;
+// chunk sums -> mean rounded to the input dtype, stored widened
+__global__ __launch_bounds__(kFinThreads) void k_mean_finalize_kernel(const float* __restrict__ part, int nch, int L,
+                                                                      int dtype, int smooth,
+                                                                      float* __restrict__ k_mean) {
+  __shared__ float s_part[kFinMaxChunks * kD];
+  const int bh = blockIdx.x;
+  const float tot = combine_partials<0>(part + (int64_t)bh * nch * kD, nch, s_part);
+  if (threadIdx.x < kD) {
+    const float mean = __fdiv_rn(tot, (float)L);
+    k_mean[bh * kD + threadIdx.x] = smooth ? round_to_half_dtype(mean, dtype) : 0.0f;
+  }
+}
+
+__global__ __launch_bounds__(kFinThreads) void v_scale_finalize_kernel(const float* __restrict__ part, int nch,
+                                                                       float* __restrict__ v_scale,
+                                                                       float* __restrict__ v_inv) {
+  __shared__ float s_part[kFinMaxChunks * kD];
+  const int bh = blockIdx.x;
+  const float amax = combine_partials<1>(part + (int64_t)bh * nch * kD, nch, s_part);
+  if (threadIdx.x < kD) {
+    const bool nz = amax > 0.0f;
+    v_scale[bh * kD + threadIdx.x] = nz ? __fdiv_rn(amax, 448.0f) : 0.0f;
+    v_inv[bh * kD + threadIdx.x] = nz ? __fdiv_rn(448.0f, amax) : 0.0f;
+  }
 }
 
 // Unnormalised Walsh-Hadamard transform of one 128-channel row held by 8 adjacent lanes x 16
@@ -348,12 +380,12 @@ hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, fl
 
 hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
                                   hipStream_t s) {
-  k_mean_finalize_kernel<<<dim3(BH), dim3(kD), 0, s>>>(part, nch, L, dtype, smooth, k_mean);
+  k_mean_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, L, dtype, smooth, k_mean);
   return hipGetLastError();
 }
 
 hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s) {
-  v_scale_finalize_kernel<<<dim3(BH), dim3(kD), 0, s>>>(part, nch, v_scale, v_inv);
+  v_scale_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, v_scale, v_inv);
   return hipGetLastError();
 }
 
