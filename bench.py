@@ -22,6 +22,9 @@ import torch
 METRIC = "Sage-attn effective TFLOPS & % INT8/FP8 MFMA peak, Wan-14B 480p (L=32760)"
 MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense INT8 (POP/s) = dense FP8 (PFLOP/s) = 5.0e15 /s
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the attention kernel at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from
+# two rocprofv3 --pmc runs, factors from a 1 GiB device copy in the same runs (profiles/sage_attn_fwd_kernel_wan14b_480p.md)
+ATTN_TRAFFIC_BYTES = {"wan14b_480p": 1808505 * 1024}
 
 
 def parse():
@@ -31,6 +34,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default=None, help="one of ksanadit_amd.workloads.WORKLOADS (default: headline)")
     ap.add_argument("--pwl-exp2", action="store_true", help="piecewise-linear e4m3 code instead of exp2 on the transcendental unit (faster, less accurate)")
+    ap.add_argument("--calib-copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (reference point for HBM traffic counters)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
     return ap.parse_args()
 
@@ -98,6 +102,12 @@ def main() -> int:
         if ev:
             ev[2].record()
 
+    if args.calib_copy_mib:
+        src = torch.empty(args.calib_copy_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads and writes calib_copy_mib MiB once each
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -143,7 +153,7 @@ def main() -> int:
             "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(attn_tflops / MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": ATTN_TRAFFIC_BYTES.get(w.name),
         },
         "quantizer_roofline": {
             "kernels": "col_partial x2, finalize x2, quant_q, quant_k, quant_v",
