@@ -225,14 +225,15 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     return max(max(max8(blk[0], 0), max8(blk[0], 8)), max(max8(blk[1], 0), max8(blk[1], 8)));
   };
   // new running max of query l32 given this lane's tile maximum; returns 2^(old max - new max)
-  auto update_max = [&](int imax, float sc) -> float {
+  auto update_max = [&](int imax, float sc, float mneg) -> float {
     {
       // the other half of query l32's keys lives in lane l32 + 32
       int other = imax;
       const auto sw = __builtin_amdgcn_permlane32_swap(imax, other, false, false);
       imax = max(sw[0], sw[1]);
     }
-    const float m_tile = (float)(imax - kMagicI) * sc;
+    // the accumulator read as fp32 is magic + dot, so one fma gives sc * dot (mneg = -magic * sc)
+    const float m_tile = __builtin_fmaf(__int_as_float(imax), sc, mneg);
     const float m_new = fmaxf(m_run, m_tile);
     const float alpha = fast_exp2(m_run - m_new);
     m_run = m_new;
@@ -307,10 +308,11 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     // row sums of tile j-1: 64 matrix cycles that run under the max finalisation below
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
     const float sc = qs * ks_cur;
-    alpha_prev = update_max(mx_cur, sc);
+    const float mneg = -kMagicF * sc;
+    alpha_prev = update_max(mx_cur, sc, mneg);
     // exponent of key r: x = sc*dot - m_run + shift, with the magic folded into the constant
     // (which is therefore off by at most ~1.5 integer steps of the dot product)
-    const float c = (kPShift - m_run) - kMagicF * sc;
+    const float c = (kPShift - m_run) + mneg;
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     v8i pf;
@@ -391,8 +393,9 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         if (key >= p.Lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
       }
     const float sc = qs * s_ks[j];
-    scale_o(update_max(lane_max(s_cur), sc));
-    const float c = (kPShift - m_run) - kMagicF * sc;
+    const float mneg = -kMagicF * sc;
+    scale_o(update_max(lane_max(s_cur), sc, mneg));
+    const float c = (kPShift - m_run) + mneg;
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     v8i pf;

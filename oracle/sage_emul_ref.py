@@ -70,7 +70,8 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 # float64) so that e4m3 codes agree except at exact rounding ties:
                 #   x_f = float(MAGIC + dot)            the int32 accumulator read as fp32
                 #   sc  = q_scale * k_scale             one fp32 product per (row, tile)
-                #   c   = (SHIFT - m) - MAGIC * sc      fp32, in this order
+                #   m   = max(m, fma(x_f_max, sc, -MAGIC * sc))
+                #   c   = (SHIFT - m) + (-MAGIC * sc)   fp32, in this order
                 #   exponent = fma(x_f, sc, c)          (pwl: fma(x_f, 8 sc, fma(8, c, 55.5)))
                 magic = 12582912.0
                 x_f = (s_int + magic).to(torch.float32)  # exact: |dot| < 2**22
@@ -82,10 +83,11 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 for j0 in range(0, Lk, BLKK):
                     sc = (qs_row[b, h][:, None] * k_scale[b, hk, j0 // BLKK]).to(torch.float32)
                     xt = x_f[:, j0 : j0 + BLKK]
-                    m_tile = (xt.amax(dim=1, keepdim=True) - magic) * sc
+                    mneg = -(magic * sc)  # fp32
+                    m_tile = (xt.amax(dim=1, keepdim=True).double() * sc.double() + mneg.double()).float()  # fma
                     m_new = torch.maximum(m, m_tile)
                     alpha = torch.exp2(m - m_new)
-                    c = (P_SHIFT - m_new) - magic * sc
+                    c = (P_SHIFT - m_new) + mneg
                     if exact_exp2:
                         e = (xt.double() * sc.double() + c.double()).float()
                         p8 = torch.exp2(e).clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
