@@ -21,6 +21,7 @@
 // int->float conversion from the softmax: p = exp2(fma(acc_as_float, sc, c)).
 #include "sage_kernels.h"
 
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/ksana_sage_hip.h"
@@ -441,11 +442,19 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 template <int DT, bool kPwlExp>
 hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
-  // more than 64 KiB of dynamic LDS has to be requested per kernel, once per process
-  static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStageBytes + kMaxKeyTiles * 4);
-  if (attr != hipSuccess) return attr;
+  // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
+  constexpr int kMaxDevices = 64;
+  static std::atomic<bool> requested[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  if (!requested[dev].load(std::memory_order_acquire)) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStageBytes + kMaxKeyTiles * 4);
+    if (e != hipSuccess) return e;
+    requested[dev].store(true, std::memory_order_release);
+  }
   sage_attn_fwd_kernel<DT, kPwlExp><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
 }

@@ -181,6 +181,9 @@ def sageattn(
         raise ValueError(f"incompatible shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
     q, k, v = _usable(q), _usable(k), _usable(v)
     B, Lq, Hq, D = q.shape
+    if q.numel() == 0:  # nothing to attend from: same empty result SDPA gives
+        out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
+        return out.transpose(1, 2) if tensor_layout == "HND" else out
     sm_scale = D**-0.5 if sm_scale is None else float(sm_scale)
     ws = workspace_for(q, k) if workspace is None else workspace
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
