@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 2
+#define KSANA_SAGE_ABI_VERSION 3
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -109,16 +109,21 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], con
 
 /* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
  * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel
- * call (sage_sla.py:237-253, dense form).  causal must be 0 in this build; flags: KSANA_SAGE_FLAG_*. */
+ * call (sage_sla.py:237-253, dense form).  causal must be 0 in this build; flags: KSANA_SAGE_FLAG_*.
+ * k_lens: NULL, or a device array of B int32: batch b attends to keys [0, k_lens[b]) only
+ * (clamped to [0, Lk]; a batch without keys gets zeros).  Same meaning as the k_lens the
+ * reference's callers pass (wan_model.py:182-189) and its variable-length backend honours
+ * (flash_attn.py:131-139); the reference's Sage adaptor drops the argument (sage_attn.py:58-84),
+ * which is what NULL reproduces.  The quantizers always see all Lk rows. */
 int ksana_sage_attn_fwd(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
-                        const ksana_sage_shape* shape, int causal, int flags, void* stream);
+                        const ksana_sage_shape* shape, const int32_t* k_lens, int causal, int flags, void* stream);
 
 /* The whole path in one call: quant_q, quant_k, quant_v, attn_fwd on `stream`.
  * Replaces sageattn(q, k, v, tensor_layout="NHD", is_causal=causal) (sage_attn.py:75-81). */
 int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype,
                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
-                       const int64_t o_strides[4], const ksana_sage_shape* shape, float sm_scale, int smooth_k,
-                       int causal, int flags, void* workspace, void* stream);
+                       const int64_t o_strides[4], const ksana_sage_shape* shape, const int32_t* k_lens,
+                       float sm_scale, int smooth_k, int causal, int flags, void* workspace, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -61,8 +61,8 @@ def _declare(lib):
     lib.ksana_sage_quant_q.argtypes, lib.ksana_sage_quant_q.restype = [vp, i, st, sp, f, vp, vp], i
     lib.ksana_sage_quant_k.argtypes, lib.ksana_sage_quant_k.restype = [vp, i, st, sp, i, vp, vp], i
     lib.ksana_sage_quant_v.argtypes, lib.ksana_sage_quant_v.restype = [vp, i, st, sp, vp, vp], i
-    lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, i, i, vp], i
-    lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, f, i, i, i, vp, vp]
+    lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, vp, i, i, vp], i
+    lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward.restype = i
 
 

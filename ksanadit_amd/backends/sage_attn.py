@@ -10,6 +10,9 @@ and ignored, as the reference's adaptor ignores them.
 Differences, all deliberate:
 * the stored ``softmax_scale`` is USED (the reference stores it and lets the callee default to
   ``D ** -0.5``; the two agree for every caller because attention_op.py:39 defaults to that value);
+* ``k_lens``: ignored by default, exactly like the reference's adaptor (sage_attn.py:58-84).  Constructed with
+  ``honor_k_lens=True`` the backend limits batch ``b`` to its first ``k_lens[b]`` keys, which is what the reference's
+  variable-length backend does with the same argument (flash_attn.py:131-139) and what padded batches need;
 * availability: no HIP device -> ``supports()`` is False and the selector moves on, like the
   reference without its package (sage_attn.py:21-27,36-38); a HIP device with a missing or stale
   library raises instead of falling back, so a broken build cannot hide behind another backend.
@@ -58,6 +61,7 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
         self.causal = causal
         self.softmax_scale = softmax_scale
         self.dropout = float(extra_impl_args.get("dropout_p", 0.0))
+        self.honor_k_lens = bool(extra_impl_args.get("honor_k_lens", False))
         self.attention_config = attention_config
         self.check_config()
 
@@ -65,5 +69,7 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
         original_dtype = query.dtype
         if original_dtype not in (torch.float16, torch.bfloat16):
             query, key, value = (t.to(torch.bfloat16) for t in (query, key, value))
-        output = sageattn(query, key, value, tensor_layout="NHD", is_causal=self.causal, sm_scale=self.softmax_scale)
+        k_lens = kwargs.get("k_lens") if self.honor_k_lens else None
+        output = sageattn(query, key, value, tensor_layout="NHD", is_causal=self.causal, sm_scale=self.softmax_scale,
+                          k_lens=k_lens)
         return output if output.dtype == original_dtype else output.to(original_dtype)

@@ -118,6 +118,19 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const int q0 = qwg * kAttnQPerWg + wave * 32;
   const bool active = q0 < p.Lq;  // wave-uniform; inactive waves only help move tiles
 
+  // keys [0, lk) of this batch take part: all of them, or the caller's per-batch count
+  int lk = p.Lk;
+  if (p.k_lens != nullptr) lk = min(max(p.k_lens[b], 0), p.Lk);  // uniform: a scalar load
+  if (lk == 0) {  // softmax over no key: the output rows are defined as zeros
+    const int q = q0 + l32;
+    if (q < p.Lq) {
+      uint4* orow = reinterpret_cast<uint4*>(p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH + 64 * hh);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) orow[i] = make_uint4(0, 0, 0, 0);
+    }
+    return;
+  }
+
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   // ---- Q fragments (B operand), 4 channel steps --------------------------------------
@@ -161,7 +174,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const uint8_t* v_src = p.v_tiles + (int64_t)bhk * p.nkb * kTileBytes;
   const unsigned copy_off = tid * 16;  // this lane's 16 bytes inside a tile
   const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb;
-  const int nkb = p.nkb;
+  const int nkb = (lk + kBlkK - 1) / kBlkK;  // tiles this batch uses; p.nkb stays the per-head stride
   // K scales live in LDS behind the ring: a per-tile global load would share the in-order
   // vmcnt queue with the tile copies and stall on all of them
   float* s_ks = reinterpret_cast<float*>(smem + kStages * kStageBytes);
@@ -171,7 +184,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   // Each wave moves its 1 KiB slice of the K tile and of the V^T tile (lane i -> byte 16*i of
   // the slice).  Copies retire in issue order, so "at most 2*n outstanding" == "all but the
   // newest n tiles have landed".
-  const bool has_tail = (p.Lk & (kBlkK - 1)) != 0;  // keys >= Lk live only in the last tile
+  const bool has_tail = (lk & (kBlkK - 1)) != 0;  // keys >= lk live only in the last tile
   const int n_main = has_tail ? nkb - 1 : nkb;       // tiles handled by the pipelined loop
   auto issue_copy = [&](int tile) {
     // clamped: past the end the last tile is copied again into a stage nobody reads any more,
@@ -383,7 +396,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_prev);
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
   }
-  if (has_tail) {  // ragged last tile, not pipelined: mask keys >= Lk
+  if (has_tail) {  // ragged last tile, not pipelined: mask keys >= lk
     const int j = nkb - 1;
     v16i (&s_cur)[2] = (n_main & 1) ? s_b : s_a;
 #pragma unroll
@@ -391,7 +404,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int key = j * kBlkK + 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
-        if (key >= p.Lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
+        if (key >= lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
       }
     const float sc = qs * s_ks[j];
     const float mneg = -kMagicF * sc;
@@ -405,12 +418,12 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int w = pack4(s_cur[t][4 * g], s_cur[t][4 * g + 1], s_cur[t][4 * g + 2], s_cur[t][4 * g + 3], scp, cp);
-        // zero the bytes of keys at or beyond Lk (code 0 is +0.0 in e4m3)
+        // zero the bytes of keys at or beyond lk (code 0 is +0.0 in e4m3)
         unsigned keep = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = j * kBlkK + 32 * t + 8 * g + 4 * hh + i;
-          if (key < p.Lk) keep |= 0xffu << (8 * i);
+          if (key < lk) keep |= 0xffu << (8 * i);
         }
         pf[4 * t + g] = w & (int)keep;
       }

@@ -173,12 +173,13 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksan
 }
 
 int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
-                        int causal, int flags, void* stream) {
+                        const int32_t* k_lens, int causal, int flags, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
   if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
+  if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
   ksana_sage_ws_layout l;
   ksana_sage_workspace_layout(s, &l);
   ksana_sage::AttnParams p;
@@ -192,14 +193,15 @@ int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4
   p.B = s->B, p.Hq = s->Hq, p.Hkv = s->Hkv, p.Lq = s->Lq, p.Lk = s->Lk;
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;
   p.exact_exp2 = (flags & KSANA_SAGE_FLAG_PWL_EXP2) ? 0 : 1;
+  p.k_lens = k_lens;
   hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
 }
 
 int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
                        const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
-                       const ksana_sage_shape* s, float sm_scale, int smooth_k, int causal, int flags, void* ws,
-                       void* stream) {
+                       const ksana_sage_shape* s, const int32_t* k_lens, float sm_scale, int smooth_k, int causal,
+                       int flags, void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
   // validate everything before the first launch so a bad argument leaves no partial work
@@ -211,7 +213,7 @@ int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int
   if (int rc = ksana_sage_quant_q(q, dtype, q_st, s, sm_scale, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_k(k, dtype, k_st, s, smooth_k, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_v(v, dtype, v_st, s, ws, stream)) return rc;
-  return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, causal, flags, stream);
+  return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, k_lens, causal, flags, stream);
 }
 
 }  // extern "C"

@@ -50,6 +50,7 @@ struct AttnParams {
   OutTensor o;
   int B, Hq, Hkv, Lq, Lk, lq_pad, nkb;
   int exact_exp2;  // 1: exp2 on the transcendental unit; 0: piecewise-linear e4m3 code (faster)
+  const int32_t* k_lens;  // optional [B]: batch b attends to keys [0, clamp(k_lens[b], 0, Lk)); nullptr = all
 };
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s);
 

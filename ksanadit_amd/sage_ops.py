@@ -145,12 +145,27 @@ def quant_v(v: torch.Tensor, ws: SageWorkspace) -> None:
     _capi.check(rc, "ksana_sage_quant_v")
 
 
-def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False) -> torch.Tensor:
+def _k_lens_arg(k_lens, batch: int, device: torch.device):
+    """``k_lens`` as the int32 device array the library reads (kept alive by the caller's reference)."""
+    if k_lens is None:
+        return None
+    k_lens = torch.as_tensor(k_lens)
+    if k_lens.dim() != 1 or k_lens.numel() != batch:
+        raise ValueError(f"k_lens must hold one length per batch entry ({batch}), got shape {tuple(k_lens.shape)}")
+    return k_lens.to(device=device, dtype=torch.int32).contiguous()
+
+
+def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False,
+             k_lens=None) -> torch.Tensor:
+    """Attention on the quantized operands in ``ws``.  ``k_lens`` (optional, one int per batch entry): batch ``b``
+    attends to keys ``[0, k_lens[b])`` only, the meaning the reference's callers give it (wan_model.py:182-189,
+    flash_attn.py:131-139); a batch entry without keys yields zeros."""
     _require_hip(out)
     lib = _capi.load()
     flags = _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0
+    kl = _k_lens_arg(k_lens, out.shape[0], out.device)
     rc = lib.ksana_sage_attn_fwd(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
-                                 int(causal), flags, _stream_ptr(out.device))
+                                 None if kl is None else kl.data_ptr(), int(causal), flags, _stream_ptr(out.device))
     _capi.check(rc, "ksana_sage_attn_fwd")
     return out
 
@@ -165,8 +180,11 @@ def sageattn(
     smooth_k: bool = True,
     workspace: SageWorkspace | None = None,
     pwl_exp2: bool = False,
+    k_lens=None,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
+
+    ``k_lens`` (optional, one int per batch entry) limits batch ``b`` to its first ``k_lens[b]`` keys.
 
     ``pwl_exp2=True`` computes the e4m3 code of every probability directly (exp2 with a
     piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate."""
@@ -188,10 +206,11 @@ def sageattn(
     ws = workspace_for(q, k) if workspace is None else workspace
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
+    kl = _k_lens_arg(k_lens, B, q.device)
     rc = lib.ksana_sage_forward(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
         _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape),
-        sm_scale, int(smooth_k), int(is_causal), _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
+        None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal), _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
     )
     _capi.check(rc, "ksana_sage_forward")
     return out.transpose(1, 2) if tensor_layout == "HND" else out

@@ -42,12 +42,13 @@ def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
 
 
 def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True,
-                         exact_exp2=True):
+                         exact_exp2=True, k_lens=None):
     """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
 
     ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
     decides where each P lands on the e4m3 grid, so the fp8 rounding of P matches the kernel's
     (a full softmax rounds P relative to the FINAL max - same accuracy, different bits).
+    ``k_lens``: batch ``b`` uses keys ``[0, k_lens[b])`` of the quantized operands (online form only).
     """
     B, H, Lq, D = q_i8.shape
     Hkv, Lk = k_i8.shape[1], k_i8.shape[2]
@@ -55,7 +56,13 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     out = torch.empty(B, Lq, H, D, dtype=out_dtype)
     qs_row = q_scale.repeat_interleave(BLKQ, dim=2)[:, :, :Lq]  # [B, H, Lq] (BLKQ == 1: already per row)
     ks_col = k_scale.repeat_interleave(BLKK, dim=2)[:, :, :Lk]  # [B, Hkv, Lk]
+    if k_lens is not None and not online:
+        raise NotImplementedError("k_lens with the full-softmax form")
     for b in range(B):
+        lk_b = Lk if k_lens is None else max(0, min(int(k_lens[b]), Lk))
+        if lk_b == 0:
+            out[b] = 0
+            continue
         for h in range(H):
             hk = h // g
             # int8 x int8 sums stay below 2**24, so fp32 matmul is exact here
@@ -80,9 +87,10 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 acc = torch.zeros(Lq, D)
                 if causal:
                     raise NotImplementedError("online emulation of causal masking")
-                for j0 in range(0, Lk, BLKK):
+                for j0 in range(0, lk_b, BLKK):
+                    j1 = min(j0 + BLKK, lk_b)
                     sc = (qs_row[b, h][:, None] * k_scale[b, hk, j0 // BLKK]).to(torch.float32)
-                    xt = x_f[:, j0 : j0 + BLKK]
+                    xt = x_f[:, j0:j1]
                     mneg = -(magic * sc)  # fp32
                     m_tile = (xt.amax(dim=1, keepdim=True).double() * sc.double() + mneg.double()).float()  # fma
                     m_new = torch.maximum(m, m_tile)
@@ -97,7 +105,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                         code = torch.round(t).clamp_(0, 126).long()
                         p8 = e4m3fn_decode_table().float()[code]
                     l = l * alpha + p8.sum(dim=1, keepdim=True)  # the normaliser sees the rounded P too
-                    acc = acc * alpha + p8 @ vf[j0 : j0 + BLKK]
+                    acc = acc * alpha + p8 @ vf[j0:j1]
                     m = m_new
                 o = acc / l * v_scale[b, hk][None, :]
             else:
@@ -109,7 +117,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     return out
 
 
-def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True, exact_exp2=True):
+def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True, exact_exp2=True, k_lens=None):
     """[B, L, H, D] half in, same out: quantise with the oracle quantizer, then emulate."""
     D = q.shape[-1]
     sm_scale = D**-0.5 if sm_scale is None else sm_scale
@@ -117,4 +125,4 @@ def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online
     k_i8, k_scale, _ = quant_k_ref(k, smooth_k=smooth_k)
     v_fp8, v_scale = quant_v_ref(v)
     return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal, online=online,
-                                exact_exp2=exact_exp2)
+                                exact_exp2=exact_exp2, k_lens=k_lens)

@@ -11,8 +11,15 @@ import torch
 import torch.nn.functional as F
 
 
-def sdpa_ref(q, k, v, *, scale=None, causal=False):
-    """``[B, L, H, D]`` in, ``[B, L, H, D]`` out, in the input dtype (sdpa.py:62-79)."""
+def sdpa_ref(q, k, v, *, scale=None, causal=False, k_lens=None):
+    """``[B, L, H, D]`` in, ``[B, L, H, D]`` out, in the input dtype (sdpa.py:62-79).
+
+    ``k_lens`` (one int per batch entry) follows the reference's variable-length backend, which cuts
+    batch ``b`` down to ``key[b, :k_lens[b]]`` / ``value[b, :k_lens[b]]`` before attending
+    (flash_attn.py:131-139); here the same keys are kept by a boolean mask.  A batch entry without
+    keys gives zeros."""
+    if k_lens is not None:
+        return _sdpa_ref_k_lens(q, k, v, scale, causal, k_lens)
     qt, kt, vt = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
     if qt.shape[1] != kt.shape[1]:
         out = F.scaled_dot_product_attention(qt, kt, vt, dropout_p=0.0, is_causal=causal, scale=scale, enable_gqa=True)
@@ -21,9 +28,27 @@ def sdpa_ref(q, k, v, *, scale=None, causal=False):
     return out.transpose(1, 2)
 
 
-def sdpa_ref_fp32(q, k, v, *, scale=None, causal=False):
+def _sdpa_ref_k_lens(q, k, v, scale, causal, k_lens):
+    if causal:
+        raise NotImplementedError("k_lens together with causal masking")
+    B, Lk = k.shape[0], k.shape[1]
+    lens = torch.as_tensor(k_lens, dtype=torch.int64).clamp(0, Lk)
+    keep = torch.arange(Lk)[None, :] < lens[:, None]  # [B, Lk]
+    qt, kt, vt = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+    gqa = qt.shape[1] != kt.shape[1]
+    out = F.scaled_dot_product_attention(qt, kt, vt, attn_mask=keep[:, None, None, :].to(q.device), dropout_p=0.0,
+                                         scale=scale, **({"enable_gqa": True} if gqa else {}))
+    out = out.transpose(1, 2)
+    empty = (lens == 0).to(q.device)
+    if bool(empty.any()):
+        out = out.clone()
+        out[empty] = 0
+    return out
+
+
+def sdpa_ref_fp32(q, k, v, *, scale=None, causal=False, k_lens=None):
     """Same computation with fp32 operands: the error budget's zero point."""
-    return sdpa_ref(q.float(), k.float(), v.float(), scale=scale, causal=causal)
+    return sdpa_ref(q.float(), k.float(), v.float(), scale=scale, causal=causal, k_lens=k_lens)
 
 
 def attention_bruteforce_f64(q, k, v, *, scale=None, causal=False):

@@ -29,11 +29,12 @@ def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
     return q.to(dtype), k.to(dtype), v.to(dtype)
 
 
-def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True):
+def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True, k_lens=None):
     """The CPU emulation fed with the operands the GPU quantizer actually produced."""
     return sage_emul_from_quant(
         ws.q_i8.cpu()[:, :, :Lq], ws.q_scale.cpu()[:, :, :Lq], untile_k(ws.k_tiles.cpu(), Lk), ws.k_scale.cpu(),
         untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), dtype, exact_exp2=exact_exp2,
+        k_lens=k_lens,
     )
 
 
@@ -129,6 +130,60 @@ def test_k_offset_invariance_and_determinism(hip_device):
     assert _cos(a.cpu(), ref) >= 0.998  # bf16 K carries only 8 bits next to an offset of 40-120
     rough = sage_ops.sageattn(*dev, smooth_k=False)
     assert _cos(rough.cpu(), ref) < _cos(a.cpu(), ref)
+
+
+@pytest.mark.parametrize("k_lens", [[300, 129], [64, 1], [0, 257], [5000, -3]])
+def test_k_lens_limits_the_keys_per_batch(hip_device, k_lens):
+    """Batch b attends to keys [0, k_lens[b]) (flash_attn.py:131-139); values are clamped to [0, Lk]; no key -> zeros."""
+    B, Lq, Lk, H = 2, 200, 300, 2
+    print(f"case k_lens={k_lens} B={B} Lq={Lq} Lk={Lk} H={H}", flush=True)
+    q, k, v = _rand_qkv(B, Lq, Lk, H, H, seed=77)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    lens_dev = torch.tensor(k_lens, device=hip_device)  # int64 on the device: converted by the wrapper
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, k_lens=lens_dev).cpu()
+    clamped = [max(0, min(n, Lk)) for n in k_lens]
+    emul = _emul_from_ws(ws, Lq, Lk, q.dtype, k_lens=clamped)
+    ref = sdpa_ref(q, k, v, k_lens=clamped)
+    for b, n in enumerate(clamped):
+        if n == 0:
+            assert (out[b] == 0).all()
+            continue
+        scale = max(emul[b].float().abs().max().item(), 1e-3)
+        assert (out[b].float() - emul[b].float()).abs().max() <= 2e-2 * scale
+        assert _cos(out[b], emul[b]) > 0.99999
+        assert (out[b].float() - ref[b].float()).abs().max() <= 0.12 * max(ref[b].float().abs().max().item(), 0.1)
+        if n >= 64:
+            assert _cos(out[b], ref[b]) >= COS_MIN
+    # the full length is the same launch as no k_lens at all, bit for bit
+    full = sage_ops.attn_fwd(ws, torch.empty_like(qd), k_lens=[Lk, Lk + 9]).cpu()
+    none = sage_ops.attn_fwd(ws, torch.empty_like(qd)).cpu()
+    assert torch.equal(full, none)
+    # rows past k_lens never reach the result: overwrite their quantized images and rerun
+    if min(clamped) >= 64:
+        out_a = sage_ops.attn_fwd(ws, torch.empty_like(qd), k_lens=clamped).cpu()
+        n_tiles_used = [(n + 63) // 64 for n in clamped]
+        for b, t in enumerate(n_tiles_used):
+            ws.k_tiles[b, :, t:] = 0x55
+            ws.v_tiles[b, :, t:] = 0x3C
+        out_b = sage_ops.attn_fwd(ws, torch.empty_like(qd), k_lens=clamped).cpu()
+        assert torch.equal(out_a, out_b)
+
+
+def test_backend_k_lens_is_opt_in(hip_device):
+    """The reference's Sage adaptor drops k_lens (sage_attn.py:58-84): so does the backend unless told otherwise."""
+    from ksanadit_amd.backends.sage_attn import SageAttentionImpl
+    q, k, v = _rand_qkv(2, 128, 192, 2, 2, seed=5)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    cfg = KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN)
+    lens = torch.tensor([100, 192], device=hip_device, dtype=torch.int32)
+    plain = SageAttentionImpl(cfg, 2, 128, False, 128**-0.5)
+    honoring = SageAttentionImpl(cfg, 2, 128, False, 128**-0.5, honor_k_lens=True)
+    base = plain.forward(qd, kd, vd).cpu()
+    assert torch.equal(plain.forward(qd, kd, vd, k_lens=lens).cpu(), base)
+    limited = honoring.forward(qd, kd, vd, k_lens=lens).cpu()
+    assert torch.equal(limited[1], base[1]) and not torch.equal(limited[0], base[0])
+    assert _cos(limited, sdpa_ref(q, k, v, k_lens=[100, 192])) >= COS_MIN
 
 
 @pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import quant_ref as qr
-from oracle.sage_emul_ref import sage_emul_ref
+from oracle.sage_emul_ref import sage_emul_from_quant, sage_emul_ref
 from oracle.sdpa_ref import attention_bruteforce_f64, sdpa_ref, sdpa_ref_fp32
 
 f32 = np.float32
@@ -295,6 +295,41 @@ def test_quant_v_properties():
     z = torch.zeros((1, 5, 1, 4), dtype=torch.bfloat16)
     z8, zs = qr.quant_v_ref(z)
     assert (z8.float() == 0).all() and (zs == 0).all()
+
+
+def test_sdpa_ref_k_lens_equals_cutting_the_batch_entries():
+    """flash_attn.py:131-139 builds batch b from key[b, :k_lens[b]]: the masked oracle must equal attention on the
+    cut tensors, entry by entry (an independent formulation: slicing instead of masking)."""
+    B, Lq, Lk, H, D = 3, 17, 40, 2, 16
+    q, k, v = _rand((B, Lq, H, D), 11).float(), _rand((B, Lk, H, D), 12).float(), _rand((B, Lk, H, D), 13).float()
+    lens = [40, 7, 0]
+    out = sdpa_ref(q, k, v, k_lens=lens)
+    for b, n in enumerate(lens):
+        if n == 0:
+            assert (out[b] == 0).all()
+        else:
+            cut = attention_bruteforce_f64(q[b : b + 1], k[b : b + 1, :n], v[b : b + 1, :n])
+            assert (out[b : b + 1].double() - cut).abs().max() < 1e-5
+    # lengths beyond Lk and below zero are clamped; GQA goes through the same mask
+    assert torch.equal(sdpa_ref(q, k, v, k_lens=[99, 7, -4]), out)
+    kk, vv = k[:, :, :1], v[:, :, :1]
+    o_g = sdpa_ref(q, kk, vv, k_lens=lens)
+    assert (o_g[1:2].double() - attention_bruteforce_f64(q[1:2], kk[1:2, :7], vv[1:2, :7])).abs().max() < 1e-5
+
+
+def test_sage_emul_k_lens_equals_emulating_the_cut_operands():
+    """On the SAME quantized operands, limiting the keys equals dropping the other keys' rows."""
+    B, L, H, D = 2, 200, 1, 128
+    q, k, v = _rand((B, L, H, D), 21), _rand((B, L, H, D), 22), _rand((B, L, H, D), 23)
+    q_i8, q_s = qr.quant_q_ref(q, D**-0.5)
+    k_i8, k_s, _ = qr.quant_k_ref(k)
+    v_f8, v_s = qr.quant_v_ref(v)
+    lens = [130, 64]
+    out = sage_emul_from_quant(q_i8, q_s, k_i8, k_s, v_f8, v_s, torch.bfloat16, k_lens=lens)
+    for b, n in enumerate(lens):
+        cut = sage_emul_from_quant(q_i8[b : b + 1], q_s[b : b + 1], k_i8[b : b + 1, :, :n], k_s[b : b + 1, :, : (n + 63) // 64],
+                                   v_f8[b : b + 1, :, :n], v_s[b : b + 1], torch.bfloat16)
+        assert torch.equal(out[b : b + 1], cut)
 
 
 # ------------------------------------------------------------------ emulation of the fused kernel
