@@ -1,0 +1,121 @@
+"""Oracle for what the Wan attention block does to Q and K before attention: RMSNorm over the
+whole token row, then the 3-axis rotary embedding.  Test infrastructure only.
+
+Restates, with torch CPU ops:
+* ``RMSNorm.float_rmsnorm`` - ksana/operations/ops.py:62-72: ``(x.float() * rsqrt(mean(x^2, -1) + eps)
+  * weight).type_as(x)``, used by ``norm_q`` / ``norm_k`` of ``WanSelfAttention`` on the ``[B, L, H*D]``
+  projections (ksana/models/wan/wan_model.py:81-90,163-165; weights are fp32, ``:82``);
+* ``rope_params`` and the three-way frequency table - wan_model.py:51-58,677-684;
+* ``apply_default_rope`` for one GPU (``sp_size == 1``) - ksana/utils/rope.py:21-24,43-58,61-128: pairs
+  ``(x[2i], x[2i+1])`` as complex128 times ``freqs[axis position, i]``, the first ``22`` pairs (for
+  D = 128) turning with the frame index, the next ``21`` with the row, the last ``21`` with the column;
+  rows at or beyond ``F*H*W`` pass unchanged; result cast back to the input dtype.
+
+One thing is FROZEN here beyond what the reference states, so that a GPU kernel can be compared
+bit for bit: the order of the fp32 sum behind ``mean(x^2)``.  The row is cut into groups of 8
+channels; accumulator ``i`` of 64 takes groups ``i, i+64, i+128, ...`` in order, adding the 8
+squares of each one after the other; the 64 accumulators are then combined by an adjacent-pair
+tree.  ``rsqrt`` is ``1 / sqrt`` with both operations correctly rounded (what torch computes on
+the CPU).  Any other order moves the statistic by ~1e-7 relative, i.e. flips about one bf16
+result in 10^5.
+
+Pinned by tests/test_prep_oracle.py: against ``torch.nn.functional.rms_norm`` (the library routine
+the reference's default configuration dispatches to), against float64 brute force, against an
+independent real-arithmetic form of the rotation, and by the rotation's invariants (pair norms,
+position 0, padding rows, angle addition).
+"""
+
+from __future__ import annotations
+
+import torch
+
+ROPE_TABLE_ROWS = 1024  # wan_model.py:679-681
+
+
+def rope_params(max_seq_len: int, dim: int, theta: float = 10000.0) -> torch.Tensor:
+    """complex128 ``[max_seq_len, dim // 2]``: ``exp(i * pos * theta^(-2j/dim))`` (wan_model.py:51-58)."""
+    assert dim % 2 == 0
+    freqs = torch.outer(
+        torch.arange(max_seq_len),
+        1.0 / torch.pow(theta, torch.arange(0, dim, 2).to(torch.float64).div(dim)),
+    )
+    return torch.polar(torch.ones_like(freqs), freqs)
+
+
+def wan_rope_table(head_dim: int, rows: int = ROPE_TABLE_ROWS) -> torch.Tensor:
+    """The model's ``freqs`` buffer: frame, row and column tables side by side (wan_model.py:676-684)."""
+    d = head_dim
+    return torch.cat(
+        [rope_params(rows, d - 4 * (d // 6)), rope_params(rows, 2 * (d // 6)), rope_params(rows, 2 * (d // 6))], dim=1
+    )
+
+
+def rope_split_sizes(half_dim: int) -> list[int]:
+    """Pairs per axis (rope.py:21-24): ``[22, 21, 21]`` for ``half_dim == 64``."""
+    return [half_dim - 2 * (half_dim // 3), half_dim // 3, half_dim // 3]
+
+
+def mean_square_ref(x: torch.Tensor) -> torch.Tensor:
+    """fp32 ``mean(x^2)`` over the last dim in the frozen order described in the module docstring."""
+    n = x.shape[-1]
+    assert n % 8 == 0
+    sq = x.float() * x.float()  # exact for fp16 / bf16 inputs
+    groups = n // 8
+    iters = (groups + 63) // 64
+    pad = iters * 64 * 8 - n
+    if pad:
+        sq = torch.cat([sq, torch.zeros(*sq.shape[:-1], pad)], dim=-1)  # adding +0.0 changes nothing
+    sq = sq.reshape(*sq.shape[:-1], iters, 64, 8)
+    acc = torch.zeros(*sq.shape[:-3], 64)
+    for it in range(iters):
+        for e in range(8):
+            acc = acc + sq[..., it, :, e]
+    width = 64
+    while width > 1:  # adjacent pairs: (0,1), (2,3), ... then pairs of pairs, ...
+        acc = acc.reshape(*acc.shape[:-1], width // 2, 2)
+        acc = acc[..., 0] + acc[..., 1]
+        width //= 2
+    return acc[..., 0] / torch.tensor(float(n), dtype=torch.float32)
+
+
+def inv_rms_ref(x: torch.Tensor, eps: float) -> torch.Tensor:
+    """``rsqrt(mean(x^2) + eps)`` per row, fp32 (ops.py:65-66)."""
+    return 1.0 / torch.sqrt(mean_square_ref(x) + torch.tensor(eps, dtype=torch.float32))
+
+
+def rmsnorm_ref(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``[..., H*D]`` half in, same out (ops.py:62-72)."""
+    r = inv_rms_ref(x, eps)[..., None]
+    return ((x.float() * r) * weight.float()).type_as(x)
+
+
+def rope_ref(x: torch.Tensor, grid_sizes, freqs: torch.Tensor) -> torch.Tensor:
+    """``[B, L, H, D]`` in, same shape and dtype out (rope.py:61-128, the ``sp_size == 1`` branch)."""
+    B, L, H, D = x.shape
+    half = D // 2
+    parts = freqs.to(torch.complex128).split(rope_split_sizes(half), dim=1)
+    out = []
+    for b, (f, h, w) in enumerate(torch.as_tensor(grid_sizes).tolist()):
+        f, h, w = int(f), int(h), int(w)
+        n = f * h * w
+        table = torch.cat(
+            [
+                parts[0][:f].view(f, 1, 1, -1).expand(f, h, w, -1),
+                parts[1][:h].view(1, h, 1, -1).expand(f, h, w, -1),
+                parts[2][:w].view(1, 1, w, -1).expand(f, h, w, -1),
+            ],
+            dim=-1,
+        ).reshape(n, 1, -1)
+        xb = torch.view_as_complex(x[b, :n].to(torch.float64).reshape(n, H, -1, 2))
+        xb = torch.view_as_real(xb * table).flatten(2)
+        out.append(torch.cat([xb, x[b, n:]]))  # float64 wins the concatenation; the cast below undoes it
+    return torch.stack(out, dim=0).type_as(x)
+
+
+def wan_prep_ref(x: torch.Tensor, weight, eps: float, grid_sizes, freqs, num_heads: int) -> torch.Tensor:
+    """``[B, L, H*D]`` projection -> ``[B, L, H, D]`` ready for attention (wan_model.py:163-174).
+    ``weight is None`` skips the norm, ``freqs is None`` the rotation."""
+    B, L, HD = x.shape
+    y = x if weight is None else rmsnorm_ref(x, weight, eps)
+    y = y.view(B, L, num_heads, HD // num_heads)
+    return y if freqs is None else rope_ref(y, grid_sizes, freqs)
