@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 3
+#define KSANA_SAGE_ABI_VERSION 4
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -77,11 +77,33 @@ typedef struct ksana_sage_ws_layout {
   uint64_t v_inv;   /* fp32  [B, Hkv, D]: 448/amax used by the V quantizer                      */
   uint64_t k_part;  /* fp32  [B, Hkv, nch, D] nch = ceil(Lk/256): chunk sums of K               */
   uint64_t v_part;  /* fp32  [B, Hkv, nch, D]: chunk abs-max of V                               */
+  uint64_t q_rms;   /* fp32  [B, Lq]: 1/sqrt(mean(q_row^2) + eps), written by the *_prep entry points */
+  uint64_t k_rms;   /* fp32  [B, Lk]: the same for the key rows                                 */
   int32_t lq_pad;
   int32_t nqb;
   int32_t nkb;
   int32_t nch;
 } ksana_sage_ws_layout;
+
+/* What WanSelfAttention.forward does to the q and k projections before it calls attention
+ * (wan_model.py:163-174), for the *_prep entry points to apply while they read q and k:
+ *   RMSNorm over the whole token row of H*D channels with an fp32 weight
+ *     (norm_q / norm_k, wan_model.py:81-90; ops.py:62-72), then
+ *   the 3-axis rotary embedding apply_default_rope(x, grid_sizes, freqs) (rope.py:61-128, one GPU).
+ * Results are rounded to the tensor's half type after each of the two steps, as the separate
+ * modules store them.  A NULL weight skips the norm of that tensor, NULL rope_freqs the rotation
+ * (WanCrossAttention, wan_model.py:236-237, norms but does not rotate). */
+typedef struct ksana_sage_prep {
+  const float* q_norm_weight;  /* device, fp32 [Hq*D], 16-byte aligned, or NULL                          */
+  const float* k_norm_weight;  /* device, fp32 [Hkv*D], 16-byte aligned, or NULL                         */
+  float norm_eps;
+  int32_t rope_rows;           /* rows of rope_freqs (1024 in the model, wan_model.py:679-681)           */
+  const double* rope_freqs;    /* device, complex128 [rope_rows, D/2] as (re, im) pairs: the model's     */
+                               /* `freqs` buffer (wan_model.py:677-684), 16-byte aligned, or NULL        */
+  const int32_t* grid_sizes;   /* HOST array [B, 3]: (frames, height, width) per batch entry; the        */
+                               /* reference reads it on the host as well (rope.py:107).  Needed with     */
+                               /* rope_freqs; B <= 16; each extent <= rope_rows; F*H*W <= L              */
+} ksana_sage_prep;
 
 /* Library identity.  No counterpart in the reference. */
 int ksana_sage_abi_version(void);
@@ -101,6 +123,16 @@ int ksana_sage_quant_q(const void* q, int dtype, const int64_t q_strides[4], con
  * (K half of sage_sla.py:202-204). */
 int ksana_sage_quant_k(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
                        int smooth_k, void* workspace, void* stream);
+
+/* quant_q / quant_k with the step before attention folded in: q and k are the projections
+ * viewed [B, L, H, D] (the H stride must be D: a token row is one contiguous run of H*D channels).
+ * Replaces norm_q/norm_k + apply_default_rope + the quantizer of the path (wan_model.py:163-174
+ * followed by sage_sla.py:198-204) without the two intermediate tensors: one extra read of the
+ * input for the row statistic instead of two writes and two reads. */
+int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t q_strides[4], const ksana_sage_shape* shape,
+                            const ksana_sage_prep* prep, float sm_scale, void* workspace, void* stream);
+int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
+                            const ksana_sage_prep* prep, int smooth_k, void* workspace, void* stream);
 
 /* V -> transposed, padded, operand-ordered fp8 e4m3fn with one fp32 scale per (b, h, d).
  * Replaces transpose_pad_permute_cuda + scale_fuse_quant_cuda (sage_sla.py:222-228). */
@@ -124,6 +156,14 @@ int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int
                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
                        const int64_t o_strides[4], const ksana_sage_shape* shape, const int32_t* k_lens,
                        float sm_scale, int smooth_k, int causal, int flags, void* workspace, void* stream);
+
+/* ksana_sage_forward with q and k taken as projections and `prep` applied on the way in
+ * (prep == NULL is ksana_sage_forward).  Replaces wan_model.py:163-174 + the attention call at :190. */
+int ksana_sage_forward_prep(const void* q, const void* k, const void* v, void* o, int dtype,
+                            const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                            const int64_t o_strides[4], const ksana_sage_shape* shape, const ksana_sage_prep* prep,
+                            const int32_t* k_lens, float sm_scale, int smooth_k, int causal, int flags,
+                            void* workspace, void* stream);
 
 #ifdef __cplusplus
 }

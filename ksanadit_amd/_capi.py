@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -26,6 +26,9 @@ EXPORTS = (
     "ksana_sage_quant_v",
     "ksana_sage_attn_fwd",
     "ksana_sage_forward",
+    "ksana_sage_quant_q_prep",
+    "ksana_sage_quant_k_prep",
+    "ksana_sage_forward_prep",
 )
 
 
@@ -38,9 +41,22 @@ class WsLayout(C.Structure):
         (n, C.c_uint64)
         for n in (
             "total_bytes", "q_i8", "q_scale", "k_i8", "k_scale", "k_mean",
-            "v_fp8", "v_scale", "v_inv", "k_part", "v_part",
+            "v_fp8", "v_scale", "v_inv", "k_part", "v_part", "q_rms", "k_rms",
         )
     ] + [(n, C.c_int32) for n in ("lq_pad", "nqb", "nkb", "nch")]
+
+
+class Prep(C.Structure):
+    """``ksana_sage_prep``: the step before attention (RMSNorm over the token row, 3-axis RoPE)."""
+
+    _fields_ = [
+        ("q_norm_weight", C.c_void_p),
+        ("k_norm_weight", C.c_void_p),
+        ("norm_eps", C.c_float),
+        ("rope_rows", C.c_int32),
+        ("rope_freqs", C.c_void_p),
+        ("grid_sizes", C.POINTER(C.c_int32)),
+    ]
 
 
 class SageLibraryError(RuntimeError):
@@ -64,6 +80,11 @@ def _declare(lib):
     lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, vp, i, i, vp], i
     lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward.restype = i
+    pp = C.POINTER(Prep)
+    lib.ksana_sage_quant_q_prep.argtypes, lib.ksana_sage_quant_q_prep.restype = [vp, i, st, sp, pp, f, vp, vp], i
+    lib.ksana_sage_quant_k_prep.argtypes, lib.ksana_sage_quant_k_prep.restype = [vp, i, st, sp, pp, i, vp, vp], i
+    lib.ksana_sage_forward_prep.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, pp, vp, f, i, i, i, vp, vp]
+    lib.ksana_sage_forward_prep.restype = i
 
 
 def library_present() -> bool:

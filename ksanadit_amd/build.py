@@ -24,6 +24,7 @@ HIPCC_FLAGS = (
     "-fPIC",
     "-shared",
     "-ffp-contract=off",  # the quantizer's arithmetic is specified to the bit; FMAs are written explicitly
+    "-fhip-fp32-correctly-rounded-divide-sqrt",  # `/` and sqrtf round correctly (hipcc's default, stated here)
     "-fno-gpu-rdc",
     # packed fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

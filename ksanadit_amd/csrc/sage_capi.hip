@@ -74,6 +74,50 @@ int check_ws(const void* ws) {
   return 0;
 }
 
+// Validates `prep` for one tensor (`weight` is that tensor's norm weight) and fills the kernel-side
+// parameters.  *out stays nullptr when there is nothing to apply.
+int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name, const int64_t st[4], int B, int L,
+              float* inv_rms, ksana_sage::PrepParams* pp, const ksana_sage::PrepParams** out) {
+  *out = nullptr;
+  if (!prep || (!weight && !prep->rope_freqs)) return 0;
+  memset(pp, 0, sizeof(*pp));
+  pp->L = L;
+  if (weight) {
+    if (reinterpret_cast<uintptr_t>(weight) & 15u)
+      return fail(KSANA_SAGE_EINVAL, "%s norm weight not 16-byte aligned", name);
+    if (st[2] != ksana_sage::kD)
+      return fail(KSANA_SAGE_EINVAL, "%s: RMSNorm over the token row needs the H stride to be %d, got %lld", name,
+                  ksana_sage::kD, (long long)st[2]);
+    if (!(prep->norm_eps >= 0.0f)) return fail(KSANA_SAGE_EINVAL, "norm_eps must be >= 0");
+    pp->inv_rms = inv_rms;
+    pp->weight = weight;
+  }
+  if (prep->rope_freqs) {
+    if (reinterpret_cast<uintptr_t>(prep->rope_freqs) & 15u)
+      return fail(KSANA_SAGE_EINVAL, "rope_freqs not 16-byte aligned");
+    if (!prep->grid_sizes) return fail(KSANA_SAGE_EINVAL, "rope_freqs given without grid_sizes");
+    if (B > ksana_sage::kMaxPrepBatch)
+      return fail(KSANA_SAGE_ENOTSUP, "RoPE on the fly supports at most %d batch entries, got %d",
+                  ksana_sage::kMaxPrepBatch, B);
+    if (prep->rope_rows < 1) return fail(KSANA_SAGE_EINVAL, "rope_rows must be positive");
+    for (int b = 0; b < B; ++b) {
+      const int32_t* g = prep->grid_sizes + 3 * b;
+      for (int a = 0; a < 3; ++a) {
+        if (g[a] < 1 || g[a] > prep->rope_rows)
+          return fail(KSANA_SAGE_EINVAL, "grid_sizes[%d][%d]=%d outside [1, rope_rows=%d]", b, a, g[a],
+                      prep->rope_rows);
+        pp->grid[b][a] = g[a];
+      }
+      if ((int64_t)g[0] * g[1] * g[2] > L)
+        return fail(KSANA_SAGE_EINVAL, "grid_sizes[%d] = %dx%dx%d exceeds the %s sequence length %d", b, g[0], g[1],
+                    g[2], name, L);
+    }
+    pp->freqs = prep->rope_freqs;
+  }
+  *out = pp;
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -109,6 +153,8 @@ int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout*
   l.v_inv = take(bhk * kD * 4);
   l.k_part = take(bhk * l.nch * kD * 4);
   l.v_part = take(bhk * l.nch * kD * 4);
+  l.q_rms = take((uint64_t)s->B * s->Lq * 4);
+  l.k_rms = take((uint64_t)s->B * s->Lk * 4);
   l.total_bytes = off;
   *out = l;
   return 0;
@@ -116,22 +162,42 @@ int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout*
 
 int ksana_sage_quant_q(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s, float sm_scale,
                        void* ws, void* stream) {
+  return ksana_sage_quant_q_prep(q, dtype, st, s, nullptr, sm_scale, ws, stream);
+}
+
+int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s,
+                            const ksana_sage_prep* prep, float sm_scale, void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("q", q, dtype, st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
   ksana_sage_ws_layout l;
   ksana_sage_workspace_layout(s, &l);
+  ksana_sage::PrepParams pp;
+  const ksana_sage::PrepParams* ppp = nullptr;
+  if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", st, s->B, s->Lq, ws_at<float>(ws, l.q_rms),
+                         &pp, &ppp))
+    return rc;
+  if (ppp && ppp->inv_rms) {
+    hipError_t e = ksana_sage::launch_row_inv_rms(in_tensor(q, dtype, st), s->B, s->Hq, s->Lq, prep->norm_eps,
+                                                  ws_at<float>(ws, l.q_rms), static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "q row statistic launch");
+  }
   // one fp32 product, then an exact power of two (1/128 undoes the unnormalised Hadamard
   // transforms of Q and K): part of the quantizer specification
   const float premul = (sm_scale * 1.4426950408889634f) * 0.0078125f;
   hipError_t e = ksana_sage::launch_quant_q(in_tensor(q, dtype, st), s->B, s->Hq, s->Lq, l.lq_pad, premul,
                                             ws_at<int8_t>(ws, l.q_i8), ws_at<float>(ws, l.q_scale),
-                                            static_cast<hipStream_t>(stream));
+                                            static_cast<hipStream_t>(stream), ppp);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_q launch");
 }
 
 int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,
                        void* ws, void* stream) {
+  return ksana_sage_quant_k_prep(k, dtype, st, s, nullptr, smooth_k, ws, stream);
+}
+
+int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
+                            const ksana_sage_prep* prep, int smooth_k, void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -140,16 +206,25 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
   hipStream_t hs = static_cast<hipStream_t>(stream);
   const ksana_sage::InTensor kt = in_tensor(k, dtype, st);
   const int bhk = s->B * s->Hkv;
+  ksana_sage::PrepParams pp;
+  const ksana_sage::PrepParams* ppp = nullptr;
+  if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", st, s->B, s->Lk, ws_at<float>(ws, l.k_rms),
+                         &pp, &ppp))
+    return rc;
   hipError_t e = hipSuccess;
+  if (ppp && ppp->inv_rms) {
+    e = ksana_sage::launch_row_inv_rms(kt, s->B, s->Hkv, s->Lk, prep->norm_eps, ws_at<float>(ws, l.k_rms), hs);
+    if (e != hipSuccess) return hip_fail(e, "k row statistic launch");
+  }
   if (smooth_k) {
-    e = ksana_sage::launch_col_partial(kt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.k_part), l.nch, hs);
+    e = ksana_sage::launch_col_partial(kt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.k_part), l.nch, hs, ppp);
     if (e != hipSuccess) return hip_fail(e, "k column-sum launch");
   }
   e = ksana_sage::launch_k_mean_finalize(ws_at<float>(ws, l.k_part), bhk, smooth_k ? l.nch : 0, s->Lk, dtype,
                                          smooth_k, ws_at<float>(ws, l.k_mean), hs);
   if (e != hipSuccess) return hip_fail(e, "k mean finalize launch");
   e = ksana_sage::launch_quant_k(kt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.k_mean),
-                                 ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs);
+                                 ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs, ppp);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_k launch");
 }
 
@@ -202,6 +277,14 @@ int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int
                        const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
                        const ksana_sage_shape* s, const int32_t* k_lens, float sm_scale, int smooth_k, int causal,
                        int flags, void* ws, void* stream) {
+  return ksana_sage_forward_prep(q, k, v, o, dtype, q_st, k_st, v_st, o_st, s, nullptr, k_lens, sm_scale, smooth_k,
+                                 causal, flags, ws, stream);
+}
+
+int ksana_sage_forward_prep(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
+                            const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
+                            const ksana_sage_shape* s, const ksana_sage_prep* prep, const int32_t* k_lens,
+                            float sm_scale, int smooth_k, int causal, int flags, void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
   // validate everything before the first launch so a bad argument leaves no partial work
@@ -210,8 +293,19 @@ int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int
   if (int rc = check_tensor("v", v, dtype, v_st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
-  if (int rc = ksana_sage_quant_q(q, dtype, q_st, s, sm_scale, ws, stream)) return rc;
-  if (int rc = ksana_sage_quant_k(k, dtype, k_st, s, smooth_k, ws, stream)) return rc;
+  if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
+  if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
+  {
+    ksana_sage::PrepParams pp;
+    const ksana_sage::PrepParams* ppp = nullptr;
+    float dummy = 0.0f;  // only the validation matters here
+    if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", q_st, s->B, s->Lq, &dummy, &pp, &ppp))
+      return rc;
+    if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", k_st, s->B, s->Lk, &dummy, &pp, &ppp))
+      return rc;
+  }
+  if (int rc = ksana_sage_quant_q_prep(q, dtype, q_st, s, prep, sm_scale, ws, stream)) return rc;
+  if (int rc = ksana_sage_quant_k_prep(k, dtype, k_st, s, prep, smooth_k, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_v(v, dtype, v_st, s, ws, stream)) return rc;
   return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, k_lens, causal, flags, stream);
 }

@@ -28,15 +28,32 @@ struct OutTensor {
   int dtype;
 };
 
+// What the Wan block does to Q and K between the projection and attention, applied by the
+// quantizer kernels to the channels they have just loaded (nullptr members switch a step off):
+// RMSNorm over the whole token row (statistic precomputed per row), then the 3-axis rotary
+// embedding with the model's complex128 table.
+constexpr int kMaxPrepBatch = 16;
+constexpr int kRopeSplit0 = 22, kRopeSplit1 = 43;  // pairs [0,22) turn with the frame, [22,43) row, [43,64) column
+struct PrepParams {
+  const float* inv_rms;  // [B, L]: 1 / sqrt(mean(x^2) + eps) of each token row; nullptr = no norm
+  const float* weight;   // [H * 128] fp32 norm weight
+  const double* freqs;   // [rows, 64] complex128 as (re, im); nullptr = no rotation
+  int L;
+  int grid[kMaxPrepBatch][3];  // (frames, height, width) per batch entry
+};
+// inv_rms[b, l] from x[b, l, :H*128] (the row must be contiguous: sH == 128)
+hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps, float* inv_rms, hipStream_t s);
+
 // column reductions over the sequence: op 0 = ordered fp32 sum, op 1 = max of |x|
-hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s);
+hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s,
+                              const PrepParams* prep = nullptr);
 hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
                                   hipStream_t s);
 hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s);
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
-                          float* q_scale, hipStream_t s);
+                          float* q_scale, hipStream_t s, const PrepParams* prep = nullptr);
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
-                          float* k_scale, hipStream_t s);
+                          float* k_scale, hipStream_t s, const PrepParams* prep = nullptr);
 hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, uint8_t* v_tiles,
                           hipStream_t s);
 

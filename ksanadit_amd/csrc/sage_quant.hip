@@ -51,14 +51,95 @@ __device__ __forceinline__ float round_to_half_dtype(float x, int dtype) {
 }
 
 // ---------------------------------------------------------------------------------------
+// The step before attention, on the 16 channels [16*c16, 16*c16+16) of head h, token `row`:
+//   y = half( (x * inv_rms[row]) * weight[ch] )                         RMSNorm, fp32, in this order
+//   (y[2i], y[2i+1]) -> half( float( (y[2i] + i*y[2i+1]) * freqs[p, i] ) )   rotation in fp64
+// with p the token's frame / row / column index for pair i in [0,22) / [22,43) / [43,64).
+// Each result is rounded to the tensor's half type exactly where a separate norm kernel and a
+// separate rotation kernel would have stored it (the fp64 product first to fp32, as a
+// conversion from double goes), so the quantizer sees the same bits.
+// Tokens at or beyond frames*height*width are normed but not rotated.
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ float through_half(float x) {
+  // The fp32 value has to exist before it is narrowed: left alone, the compiler merges the
+  // multiply that produced it with the conversion (v_fma_mixlo_f16), which rounds once
+  // instead of twice and so differs from "compute in fp32, then store as half" in rare ties.
+  asm volatile("" : "+v"(x));
+  if constexpr (DT == KSANA_SAGE_BF16) return (float)(__bf16)x;
+  return (float)(_Float16)x;
+}
+
+template <int DT>
+__device__ __forceinline__ void prep16(float* x, const PrepParams& pp, int b, int row, int h, int c16) {
+  if (pp.inv_rms != nullptr) {
+    const float r = pp.inv_rms[(int64_t)b * pp.L + row];
+    const float4* w4 = reinterpret_cast<const float4*>(pp.weight + h * kD + c16 * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float4 w = w4[j];
+      x[4 * j + 0] = through_half<DT>((x[4 * j + 0] * r) * w.x);
+      x[4 * j + 1] = through_half<DT>((x[4 * j + 1] * r) * w.y);
+      x[4 * j + 2] = through_half<DT>((x[4 * j + 2] * r) * w.z);
+      x[4 * j + 3] = through_half<DT>((x[4 * j + 3] * r) * w.w);
+    }
+  }
+  if (pp.freqs != nullptr) {
+    const int gh = pp.grid[b][1], gw = pp.grid[b][2];
+    const int plane = gh * gw;
+    if (row < pp.grid[b][0] * plane) {
+      const int f = row / plane, rem = row - f * plane;
+      const int hi = rem / gw, wi = rem - hi * gw;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int i = c16 * 8 + j;
+        const int tr = i < kRopeSplit0 ? f : (i < kRopeSplit1 ? hi : wi);
+        const double2 cs = *reinterpret_cast<const double2*>(pp.freqs + ((int64_t)tr * (kD / 2) + i) * 2);
+        const double a = (double)x[2 * j], bb = (double)x[2 * j + 1];
+        const double re = a * cs.x - bb * cs.y;
+        const double im = a * cs.y + bb * cs.x;
+        x[2 * j] = through_half<DT>((float)re);
+        x[2 * j + 1] = through_half<DT>((float)im);
+      }
+    }
+  }
+}
+
+// 1 / sqrt(mean(x^2) + eps) of every token row x[b, l, 0 : n8*8].  One wave per row: lane i takes the
+// groups of 8 channels i, i+64, i+128, ... in order, adding the 8 squares of each one after the other
+// (fp32, squares of half values are exact); the 64 lane sums meet in an adjacent-pair tree.  The order
+// is part of the result.  grid = (ceil(L / 4), B), 256 threads.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
+                                                               int L, int n8, float n_channels, float eps,
+                                                               float* __restrict__ inv_rms) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), b = blockIdx.y;
+  if (row >= L) return;
+  const uint16_t* base = x + b * sB + (int64_t)row * sL;
+  float acc = 0.0f;
+  for (int g = lane; g < n8; g += 64) {
+    float v[8];
+    widen8<DT>(*reinterpret_cast<const uint4*>(base + g * 8), v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = acc + v[e] * v[e];
+  }
+#pragma unroll
+  for (int m = 1; m <= 32; m <<= 1) acc = acc + __shfl_xor(acc, m);
+  // sqrtf, not __fsqrt_rn: the latter is the 1-ulp native instruction in this toolchain, the former is
+  // correctly rounded (the build passes -fhip-fp32-correctly-rounded-divide-sqrt)
+  if (lane == 0) inv_rms[(int64_t)b * L + row] = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(acc, n_channels) + eps));
+}
+
+// ---------------------------------------------------------------------------------------
 // Column reduction over a chunk of 256 rows.  OP 0: fp32 sum in the frozen order (slot i%32
 // sequential over the chunk's 8 row groups, then an adjacent-pair tree over the 32 slots).
 // OP 1: max |x| (order free).  grid = (nch, H, B).
 // ---------------------------------------------------------------------------------------
-template <int DT, int OP>
+template <int DT, int OP, bool PRE>
 __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
                                                                int64_t sH, int H, int L, float* __restrict__ part,
-                                                               int nch) {
+                                                               int nch, const PrepParams pp) {
   const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const uint16_t* base = x + b * sB + h * sH + c16 * 16;
@@ -67,6 +148,9 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
   for (int i = 0; i < kMeanChunk / kSlots; ++i) {
     const int row = ch * kMeanChunk + i * kSlots + slot;
     load_row16<DT>(base + (int64_t)row * sL, row < L, rows[i]);
+    if constexpr (PRE) {
+      if (row < L) prep16<DT>(rows[i], pp, b, row, h, c16);
+    }
   }
   float acc[16];
 #pragma unroll
@@ -211,10 +295,11 @@ __device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
 // workgroup handles 128 rows (4 per row slot).  grid = (lq_pad/128, H, B).  Output row-major
 // int8 [B, H, lq_pad, 128] and fp32 [B, H, lq_pad]; rows at or beyond L come out as zeros.
 // ---------------------------------------------------------------------------------------
-template <int DT>
+template <int DT, bool PRE>
 __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __restrict__ q, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L, int lq_pad, float premul,
-                                                           int8_t* __restrict__ q_i8, float* __restrict__ q_scale) {
+                                                           int8_t* __restrict__ q_i8, float* __restrict__ q_scale,
+                                                           const PrepParams pp) {
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const uint16_t* base = q + b * sB + h * sH + c16 * 16;
@@ -225,6 +310,9 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
   for (int i = 0; i < R; ++i) {
     const int row = blk * kRowsPerWg + i * kSlots + slot;
     load_row16<DT>(base + (int64_t)row * sL, row < L, x[i]);
+    if constexpr (PRE) {
+      if (row < L) prep16<DT>(x[i], pp, b, row, h, c16);
+    }
   }
 #pragma unroll
   for (int i = 0; i < R; ++i) {
@@ -251,11 +339,12 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
 // the attention kernel's int8 MFMA consumes it: fragment (t = row/32, s = 32-channel step)
 // is 64 lanes x 16 bytes, lane = 32*(16-channel half within the step) + row%32.
 // ---------------------------------------------------------------------------------------
-template <int DT>
+template <int DT, bool PRE>
 __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L, int nkb,
                                                            const float* __restrict__ k_mean,
-                                                           int8_t* __restrict__ k_tiles, float* __restrict__ k_scale) {
+                                                           int8_t* __restrict__ k_tiles, float* __restrict__ k_scale,
+                                                           const PrepParams pp) {
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const int64_t bh = (int64_t)b * H + h;
@@ -271,6 +360,9 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
     const int row = blk * kBlkK + i * kSlots + slot;
     const bool valid = row < L;
     load_row16<DT>(base + (int64_t)row * sL, valid, x[i]);
+    if constexpr (PRE) {
+      if (valid) prep16<DT>(x[i], pp, b, row, h, c16);
+    }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       x[i][e] = valid ? x[i][e] - km[e] : 0.0f;
@@ -367,13 +459,24 @@ __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __res
     }                                            \
   } while (0)
 
-hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s) {
+hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps, float* inv_rms, hipStream_t s) {
+  const dim3 grid((L + 3) / 4, B), block(kThreads);
+  KSANA_DISPATCH_DT(x.dtype, (row_inv_rms_kernel<DT><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, L, H * kD / 8,
+                                                                            (float)(H * kD), eps, inv_rms)));
+  return hipGetLastError();
+}
+
+hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s,
+                              const PrepParams* prep) {
   const dim3 grid(nch, H, B), block(kThreads);
+  const PrepParams none{};
   KSANA_DISPATCH_DT(x.dtype, {
-    if (op == 0)
-      col_partial_kernel<DT, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch);
+    if (op != 0)
+      col_partial_kernel<DT, 1, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none);
+    else if (prep == nullptr)
+      col_partial_kernel<DT, 0, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none);
     else
-      col_partial_kernel<DT, 1><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch);
+      col_partial_kernel<DT, 0, true><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, *prep);
   });
   return hipGetLastError();
 }
@@ -390,19 +493,32 @@ hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_
 }
 
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
-                          float* q_scale, hipStream_t s) {
+                          float* q_scale, hipStream_t s, const PrepParams* prep) {
   const dim3 grid(lq_pad / 128, H, B), block(kThreads);
-  KSANA_DISPATCH_DT(q.dtype,
-                    (quant_q_kernel<DT><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8,
-                                                               q_scale)));
+  const PrepParams none{};
+  KSANA_DISPATCH_DT(q.dtype, {
+    if (prep == nullptr)
+      quant_q_kernel<DT, false><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
+                                                        none);
+    else
+      quant_q_kernel<DT, true><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
+                                                       *prep);
+  });
   return hipGetLastError();
 }
 
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
-                          float* k_scale, hipStream_t s) {
+                          float* k_scale, hipStream_t s, const PrepParams* prep) {
   const dim3 grid(nkb, H, B), block(kThreads);
-  KSANA_DISPATCH_DT(k.dtype, (quant_k_kernel<DT><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean,
-                                                                         k_tiles, k_scale)));
+  const PrepParams none{};
+  KSANA_DISPATCH_DT(k.dtype, {
+    if (prep == nullptr)
+      quant_k_kernel<DT, false><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
+                                                        none);
+    else
+      quant_k_kernel<DT, true><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
+                                                       *prep);
+  });
   return hipGetLastError();
 }
 

@@ -112,27 +112,101 @@ class SageWorkspace:
         return self._view(l.v_scale, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
 
 
+    @property
+    def q_rms(self):
+        s, l = self.shape, self.layout
+        return self._view(l.q_rms, s.B * s.Lq * 4, torch.float32, (s.B, s.Lq))
+
+    @property
+    def k_rms(self):
+        s, l = self.shape, self.layout
+        return self._view(l.k_rms, s.B * s.Lk * 4, torch.float32, (s.B, s.Lk))
+
+
+@dataclass
+class WanPrep:
+    """What ``WanSelfAttention.forward`` does to the q and k projections before attention
+    (ksana/models/wan/wan_model.py:163-174), handed to the quantizer to apply while it reads them:
+    RMSNorm over the whole token row with fp32 weights (``norm_q.weight`` / ``norm_k.weight``; ``None`` skips it),
+    then ``apply_default_rope(x, grid_sizes, freqs)`` (ksana/utils/rope.py:61-128; ``freqs=None`` skips it, as in
+    the cross-attention block).  ``freqs`` is the model's complex128 buffer ``[1024, D/2]``, ``grid_sizes`` one
+    ``(frames, height, width)`` per batch entry."""
+
+    q_norm_weight: torch.Tensor | None = None
+    k_norm_weight: torch.Tensor | None = None
+    eps: float = 1e-6
+    freqs: torch.Tensor | None = None
+    grid_sizes: object = None
+
+    def to_c(self, device):
+        """The C struct plus the objects that must outlive the call."""
+        keep = []
+
+        def weight(w):
+            if w is None:
+                return None
+            w = w.to(device=device, dtype=torch.float32).contiguous()
+            keep.append(w)
+            return w.data_ptr()
+
+        c = _capi.Prep()
+        c.q_norm_weight, c.k_norm_weight = weight(self.q_norm_weight), weight(self.k_norm_weight)
+        c.norm_eps = float(self.eps)
+        if self.freqs is not None:
+            if self.freqs.dim() != 2 or not self.freqs.is_complex():
+                raise ValueError("freqs must be a complex [rows, D/2] tensor")
+            if self.grid_sizes is None:
+                raise ValueError("freqs given without grid_sizes")
+            fr = self.freqs.to(device=device, dtype=torch.complex128).contiguous()
+            grid = torch.as_tensor(self.grid_sizes).to(device="cpu", dtype=torch.int32).contiguous()
+            if grid.dim() != 2 or grid.shape[1] != 3:
+                raise ValueError(f"grid_sizes must be [B, 3], got {tuple(grid.shape)}")
+            keep += [fr, grid]
+            c.rope_freqs, c.rope_rows = fr.data_ptr(), fr.shape[0]
+            c.grid_sizes = C.cast(grid.data_ptr(), C.POINTER(C.c_int32))
+        return c, keep
+
+
+def _as_heads(x: torch.Tensor, num_heads: int | None) -> torch.Tensor:
+    """``[B, L, H*D]`` projection -> ``[B, L, H, D]`` view (4-D tensors pass through)."""
+    if x.dim() == 4:
+        return x
+    if x.dim() != 3 or num_heads is None or x.shape[-1] % num_heads:
+        raise ValueError("a projection must be [B, L, H*D] with num_heads given, or already [B, L, H, D]")
+    return x.view(x.shape[0], x.shape[1], num_heads, x.shape[-1] // num_heads)
+
+
 def workspace_for(q: torch.Tensor, k: torch.Tensor) -> SageWorkspace:
     B, Lq, Hq, D = q.shape
     _, Lk, Hkv, _ = k.shape
     return SageWorkspace.allocate(B, Hq, Hkv, Lq, Lk, D, q.device)
 
 
-def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float) -> None:
+def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: WanPrep | None = None) -> None:
     _require_hip(q)
     q = _usable(q)
     lib = _capi.load()
-    rc = lib.ksana_sage_quant_q(q.data_ptr(), _DTYPES[q.dtype], _strides(q), C.byref(ws.shape), sm_scale, ws.ptr,
-                                _stream_ptr(q.device))
+    if prep is None:
+        rc = lib.ksana_sage_quant_q(q.data_ptr(), _DTYPES[q.dtype], _strides(q), C.byref(ws.shape), sm_scale, ws.ptr,
+                                    _stream_ptr(q.device))
+    else:
+        c_prep, _keep = prep.to_c(q.device)
+        rc = lib.ksana_sage_quant_q_prep(q.data_ptr(), _DTYPES[q.dtype], _strides(q), C.byref(ws.shape),
+                                         C.byref(c_prep), sm_scale, ws.ptr, _stream_ptr(q.device))
     _capi.check(rc, "ksana_sage_quant_q")
 
 
-def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True) -> None:
+def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: WanPrep | None = None) -> None:
     _require_hip(k)
     k = _usable(k)
     lib = _capi.load()
-    rc = lib.ksana_sage_quant_k(k.data_ptr(), _DTYPES[k.dtype], _strides(k), C.byref(ws.shape), int(smooth_k), ws.ptr,
-                                _stream_ptr(k.device))
+    if prep is None:
+        rc = lib.ksana_sage_quant_k(k.data_ptr(), _DTYPES[k.dtype], _strides(k), C.byref(ws.shape), int(smooth_k),
+                                    ws.ptr, _stream_ptr(k.device))
+    else:
+        c_prep, _keep = prep.to_c(k.device)
+        rc = lib.ksana_sage_quant_k_prep(k.data_ptr(), _DTYPES[k.dtype], _strides(k), C.byref(ws.shape),
+                                         C.byref(c_prep), int(smooth_k), ws.ptr, _stream_ptr(k.device))
     _capi.check(rc, "ksana_sage_quant_k")
 
 
@@ -181,10 +255,13 @@ def sageattn(
     workspace: SageWorkspace | None = None,
     pwl_exp2: bool = False,
     k_lens=None,
+    prep: WanPrep | None = None,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
 
     ``k_lens`` (optional, one int per batch entry) limits batch ``b`` to its first ``k_lens[b]`` keys.
+    ``prep`` (optional, "NHD" only): q and k are the raw projections and the block's RMSNorm + RoPE are applied
+    while they are read (see ``WanPrep``).
 
     ``pwl_exp2=True`` computes the e4m3 code of every probability directly (exp2 with a
     piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate."""
@@ -193,6 +270,8 @@ def sageattn(
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("sageattn expects 4-D tensors")
     if tensor_layout == "HND":
+        if prep is not None:
+            raise ValueError("prep needs the NHD layout (a token row must be contiguous)")
         q, k, v = (t.transpose(1, 2) for t in (q, k, v))
     _require_hip(q, k, v)
     if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
@@ -207,10 +286,20 @@ def sageattn(
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)
-    rc = lib.ksana_sage_forward(
+    c_prep, _keep = (None, None) if prep is None else prep.to_c(q.device)
+    rc = lib.ksana_sage_forward_prep(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
         _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape),
-        None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal), _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
+        None if c_prep is None else C.byref(c_prep), None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal), _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
     )
-    _capi.check(rc, "ksana_sage_forward")
+    _capi.check(rc, "ksana_sage_forward_prep" if prep is not None else "ksana_sage_forward")
     return out.transpose(1, 2) if tensor_layout == "HND" else out
+
+
+def wan_self_attention(q_proj: torch.Tensor, k_proj: torch.Tensor, v_proj: torch.Tensor, num_heads: int,
+                       prep: WanPrep, **kwargs) -> torch.Tensor:
+    """The attention part of ``WanSelfAttention.forward`` from the three projections ``[B, L, H*D]`` on:
+    norm_q / norm_k, RoPE, attention (ksana/models/wan/wan_model.py:163-190) -> ``[B, L, H, D]``.
+    The normed and rotated q and k are never written to memory."""
+    q, k, v = (_as_heads(t, num_heads) for t in (q_proj, k_proj, v_proj))
+    return sageattn(q, k, v, tensor_layout="NHD", prep=prep, **kwargs)

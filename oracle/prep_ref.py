@@ -15,8 +15,8 @@ One thing is FROZEN here beyond what the reference states, so that a GPU kernel 
 bit for bit: the order of the fp32 sum behind ``mean(x^2)``.  The row is cut into groups of 8
 channels; accumulator ``i`` of 64 takes groups ``i, i+64, i+128, ...`` in order, adding the 8
 squares of each one after the other; the 64 accumulators are then combined by an adjacent-pair
-tree.  ``rsqrt`` is ``1 / sqrt`` with both operations correctly rounded (what torch computes on
-the CPU).  Any other order moves the statistic by ~1e-7 relative, i.e. flips about one bf16
+tree.  ``rsqrt`` is ``1 / sqrt`` with both operations correctly rounded: what ``torch.rsqrt`` computes
+on the CPU (``torch.sqrt`` does not always round correctly there, so the two are taken from numpy).  Any other order moves the statistic by ~1e-7 relative, i.e. flips about one bf16
 result in 10^5.
 
 Pinned by tests/test_prep_oracle.py: against ``torch.nn.functional.rms_norm`` (the library routine
@@ -27,6 +27,7 @@ position 0, padding rows, angle addition).
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 ROPE_TABLE_ROWS = 1024  # wan_model.py:679-681
@@ -80,7 +81,8 @@ def mean_square_ref(x: torch.Tensor) -> torch.Tensor:
 
 def inv_rms_ref(x: torch.Tensor, eps: float) -> torch.Tensor:
     """``rsqrt(mean(x^2) + eps)`` per row, fp32 (ops.py:65-66)."""
-    return 1.0 / torch.sqrt(mean_square_ref(x) + torch.tensor(eps, dtype=torch.float32))
+    t = (mean_square_ref(x) + torch.tensor(eps, dtype=torch.float32)).numpy()
+    return torch.from_numpy((np.float32(1.0) / np.sqrt(t)).astype(np.float32))
 
 
 def rmsnorm_ref(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:

@@ -30,7 +30,8 @@ def test_library_exports_every_declared_symbol():
     header = (ROOT / "include" / "ksana_sage_hip.h").read_text()
     declared = set(re.findall(r"\b(ksana_sage_[a-z_0-9]+)\s*\(", header))
     assert declared >= {"ksana_sage_forward", "ksana_sage_attn_fwd", "ksana_sage_quant_q", "ksana_sage_quant_k",
-                        "ksana_sage_quant_v", "ksana_sage_workspace_layout", "ksana_sage_last_error", "ksana_sage_abi_version"}
+                        "ksana_sage_quant_v", "ksana_sage_workspace_layout", "ksana_sage_last_error", "ksana_sage_abi_version",
+                        "ksana_sage_quant_q_prep", "ksana_sage_quant_k_prep", "ksana_sage_forward_prep"}
     lib = C.CDLL(str(_capi.LIB_PATH))
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
@@ -81,6 +82,18 @@ def test_entry_points_validate_before_touching_the_gpu():
     assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), null, 0, 0x10, null) == _capi.EINVAL  # flags
     assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), C.c_void_p(0x1002), 0, 0, null) == _capi.EINVAL  # k_lens alignment
     assert lib.ksana_sage_forward(fake, fake, null, fake, _capi.BF16, st, st, st, st, C.byref(shape), null, 0.1, 1, 0, 0, fake, null) == _capi.EINVAL
+    # the step-before-attention descriptor is validated on the host as well
+    prep = _capi.Prep()
+    prep.q_norm_weight, prep.norm_eps = 0x1004, 1e-6  # misaligned weight
+    assert lib.ksana_sage_quant_q_prep(fake, _capi.BF16, st, C.byref(shape), C.byref(prep), 0.1, fake, null) == _capi.EINVAL
+    assert b"16-byte aligned" in lib.ksana_sage_last_error()
+    prep = _capi.Prep()
+    prep.rope_freqs, prep.rope_rows = 0x1000, 1024  # rotation without a grid
+    assert lib.ksana_sage_quant_k_prep(fake, _capi.BF16, st, C.byref(shape), C.byref(prep), 1, fake, null) == _capi.EINVAL
+    grid = (C.c_int32 * 3)(2, 8, 8)  # 128 positions, 64 rows
+    prep.grid_sizes = C.cast(grid, C.POINTER(C.c_int32))
+    assert lib.ksana_sage_quant_k_prep(fake, _capi.BF16, st, C.byref(shape), C.byref(prep), 1, fake, null) == _capi.EINVAL
+    assert b"exceeds" in lib.ksana_sage_last_error()
     with pytest.raises(ValueError):
         _capi.check(_capi.EINVAL, "x")
     with pytest.raises(NotImplementedError):

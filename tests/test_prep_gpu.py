@@ -1,0 +1,123 @@
+"""The quantizer with the block's RMSNorm + RoPE folded in (through the C ABI) against
+oracle/prep_ref.py followed by oracle/quant_ref.py: every integer and every scale bit for bit."""
+
+import pytest
+import torch
+
+from ksanadit_amd import sage_ops
+from ksanadit_amd.layout import untile_k
+from ksanadit_amd.sage_ops import WanPrep
+from oracle import prep_ref as pr
+from oracle import quant_ref as qr
+from oracle.sdpa_ref import sdpa_ref
+
+pytestmark = pytest.mark.gpu
+
+
+def _proj(B, L, H, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    x = 1.5 * torch.randn((B, L, H * 128), generator=g) + 0.7 * torch.randn((1, 1, H * 128), generator=g)
+    w = 1.0 + 0.2 * torch.randn(H * 128, generator=g)
+    return x.to(dtype), w.float()
+
+
+def _check_q(ws, ref4d, sm_scale, Lq):
+    q_i8, q_scale = qr.quant_q_ref(ref4d, sm_scale)
+    assert torch.equal(ws.q_i8.cpu()[:, :, :Lq], q_i8)
+    assert torch.equal(ws.q_scale.cpu()[:, :, :Lq], q_scale)
+
+
+def _check_k(ws, ref4d, Lk):
+    k_i8, k_scale, k_mean = qr.quant_k_ref(ref4d)
+    assert torch.equal(ws.k_mean.cpu(), k_mean)
+    assert torch.equal(ws.k_scale.cpu(), k_scale)
+    assert torch.equal(untile_k(ws.k_tiles.cpu(), Lk), k_i8)
+
+
+@pytest.mark.parametrize(
+    "B,L,H,grids,dtype,norm,rope",
+    [
+        (1, 24, 2, [(2, 3, 4)], torch.bfloat16, True, True),
+        (1, 300, 12, [(3, 9, 11)], torch.bfloat16, True, True),      # 297 of 300 rows rotate, 3 pass through
+        (2, 130, 3, [(2, 5, 13), (1, 7, 9)], torch.bfloat16, True, True),
+        (1, 200, 40, [(2, 10, 10)], torch.bfloat16, True, True),     # the 14B row: 5120 channels
+        (1, 96, 4, [(1, 8, 12)], torch.float16, True, True),
+        (1, 96, 4, [(1, 8, 12)], torch.bfloat16, True, False),       # cross-attention: norm only
+        (1, 96, 4, [(4, 4, 6)], torch.bfloat16, False, True),        # rotation only
+    ],
+)
+def test_quantizer_with_prep_is_bit_exact(hip_device, B, L, H, grids, dtype, norm, rope):
+    print(f"case B={B} L={L} H={H} grids={grids} dtype={dtype} norm={norm} rope={rope}", flush=True)
+    qp, wq = _proj(B, L, H, seed=L + H, dtype=dtype)
+    kp, wk = _proj(B, L, H, seed=L + H + 1, dtype=dtype)
+    table = pr.wan_rope_table(128)
+    prep = WanPrep(q_norm_weight=wq if norm else None, k_norm_weight=wk if norm else None, eps=1e-6,
+                   freqs=table if rope else None, grid_sizes=grids if rope else None)
+    q4 = qp.view(B, L, H, 128).to(hip_device)
+    k4 = kp.view(B, L, H, 128).to(hip_device)
+    ws = sage_ops.workspace_for(q4, k4)
+    ws.blob.fill_(0x7F)
+    sage_ops.quant_q(q4, ws, 128**-0.5, prep=prep)
+    sage_ops.quant_k(k4, ws, prep=prep)
+    torch.cuda.synchronize()
+    if norm:
+        assert torch.equal(ws.q_rms.cpu(), pr.inv_rms_ref(qp, 1e-6))
+        assert torch.equal(ws.k_rms.cpu(), pr.inv_rms_ref(kp, 1e-6))
+    q_ref = pr.wan_prep_ref(qp, wq if norm else None, 1e-6, grids, table if rope else None, H)
+    k_ref = pr.wan_prep_ref(kp, wk if norm else None, 1e-6, grids, table if rope else None, H)
+    _check_q(ws, q_ref, 128**-0.5, L)
+    _check_k(ws, k_ref, L)
+
+
+def test_wan_block_path_equals_attention_on_prepared_tensors(hip_device):
+    """norm + RoPE on the fly, then attention == attention fed with the oracle's normed and rotated q, k."""
+    B, L, H = 1, 448, 6
+    grids = [(2, 14, 16)]
+    qp, wq = _proj(B, L, H, 1)
+    kp, wk = _proj(B, L, H, 2)
+    vp, _ = _proj(B, L, H, 3)
+    table = pr.wan_rope_table(128)
+    prep = WanPrep(wq, wk, 1e-6, table, grids)
+    fused = sage_ops.wan_self_attention(qp.to(hip_device), kp.to(hip_device), vp.to(hip_device), H, prep).cpu()
+    q_ref = pr.wan_prep_ref(qp, wq, 1e-6, grids, table, H)
+    k_ref = pr.wan_prep_ref(kp, wk, 1e-6, grids, table, H)
+    v4 = vp.view(B, L, H, 128)
+    plain = sage_ops.sageattn(q_ref.to(hip_device), k_ref.to(hip_device), v4.to(hip_device)).cpu()
+    assert torch.equal(fused, plain)
+    ref = sdpa_ref(q_ref, k_ref, v4)
+    a, b = fused.double().flatten(), ref.double().flatten()
+    assert float((a @ b) / (a.norm() * b.norm())) >= 0.999
+
+
+def test_prep_at_model_row_width_and_length(hip_device):
+    """Wan-14B rows (40 heads) over 4096 tokens of a 4 x 32 x 32 grid: still every bit."""
+    B, L, H = 1, 4096, 40
+    grids = [(4, 32, 32)]
+    qp, wq = _proj(B, L, H, 11)
+    kp, wk = _proj(B, L, H, 12)
+    table = pr.wan_rope_table(128)
+    prep = WanPrep(wq, wk, 1e-6, table, grids)
+    q4, k4 = qp.view(B, L, H, 128).to(hip_device), kp.view(B, L, H, 128).to(hip_device)
+    ws = sage_ops.workspace_for(q4, k4)
+    sage_ops.quant_q(q4, ws, 128**-0.5, prep=prep)
+    sage_ops.quant_k(k4, ws, prep=prep)
+    torch.cuda.synchronize()
+    assert torch.equal(ws.q_rms.cpu(), pr.inv_rms_ref(qp, 1e-6))
+    _check_q(ws, pr.wan_prep_ref(qp, wq, 1e-6, grids, table, H), 128**-0.5, L)
+    _check_k(ws, pr.wan_prep_ref(kp, wk, 1e-6, grids, table, H), L)
+
+
+def test_prep_argument_errors(hip_device):
+    qp, wq = _proj(1, 64, 2, 5)
+    q4 = qp.view(1, 64, 2, 128).to(hip_device)
+    ws = sage_ops.workspace_for(q4, q4)
+    table = pr.wan_rope_table(128)
+    with pytest.raises(ValueError, match="exceeds"):
+        sage_ops.quant_q(q4, ws, 0.1, prep=WanPrep(wq, wq, 1e-6, table, [(2, 8, 8)]))  # 128 positions > 64 rows
+    with pytest.raises(ValueError, match="outside"):
+        sage_ops.quant_q(q4, ws, 0.1, prep=WanPrep(wq, wq, 1e-6, table[:4], [(8, 2, 2)]))  # frame 8 > 4 table rows
+    with pytest.raises(ValueError, match="H stride"):
+        wide = torch.zeros(1, 64, 2, 256, dtype=torch.bfloat16, device=hip_device)[..., :128]  # heads not adjacent
+        sage_ops.quant_q(wide, ws, 0.1, prep=WanPrep(wq, wq, 1e-6, None, None))
+    with pytest.raises(ValueError, match="grid_sizes"):
+        WanPrep(wq, wq, 1e-6, table, None).to_c(hip_device)

@@ -69,6 +69,17 @@ def test_rmsnorm_against_library_routine_and_float64(dtype):
     assert ((mine.double() - exact).abs() <= 0.51 * ulp * exact.abs().clamp(min=2.0**-14) + 1e-7).all()
 
 
+def test_inv_rms_is_the_references_rsqrt():
+    """ops.py:66 calls torch.rsqrt: on the CPU that is 1/sqrt with both steps correctly rounded, which is how the
+    oracle (and the kernel) compute it."""
+    x = _half((512, 1536), 21, scale=0.8)
+    ms = pr.mean_square_ref(x)
+    want = torch.rsqrt(ms + torch.tensor(1e-6, dtype=torch.float32))
+    assert torch.equal(pr.inv_rms_ref(x, 1e-6), want)
+    exact = 1.0 / torch.sqrt(ms.double() + float(torch.tensor(1e-6, dtype=torch.float32)))
+    assert ((want.double() - exact).abs() / exact).max() < 1.2e-7
+
+
 def test_rmsnorm_invariants():
     x = _half((8, 1536), 9)
     w = torch.ones(1536)
