@@ -71,6 +71,86 @@ def cpu_baseline(workload, target_s: float):
     }
 
 
+# (frames, height, width) of the latent token grid behind each Wan workload's sequence length
+WAN_GRIDS = {"cpu_plumbing": (3, 20, 26), "wan5b_720p": (31, 22, 40), "wan14b_480p": (21, 30, 52),
+             "wan14b_720p": (21, 45, 80)}
+
+
+def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
+    """Outside the timed step: the quantizer with the block's RMSNorm + RoPE applied on the fly
+    (q and k taken as the raw projections).  Same 9 N algorithmic bytes as the plain quantizer; what a
+    separate norm kernel and a separate rotation kernel would add is 8 N more for each of q and k."""
+    g = torch.Generator().manual_seed(7)
+    wq = (1.0 + 0.2 * torch.randn(w.H * w.D, generator=g)).to(dev)
+    wk = (1.0 + 0.2 * torch.randn(w.H * w.D, generator=g)).to(dev)
+    d = w.D
+
+    def table(rows, dim):  # exp(i * pos * theta^(-2j/dim)), complex128
+        f = torch.outer(torch.arange(rows), 1.0 / torch.pow(10000.0, torch.arange(0, dim, 2).to(torch.float64).div(dim)))
+        return torch.polar(torch.ones_like(f), f)
+
+    freqs = torch.cat([table(1024, d - 4 * (d // 6)), table(1024, 2 * (d // 6)), table(1024, 2 * (d // 6))], dim=1).to(dev)
+    prep = sage_ops.WanPrep(wq, wk, 1e-6, freqs, [grid])
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
+
+    def run(e=None):
+        if e:
+            e[0].record()
+        sage_ops.quant_q(q, ws, sm_scale, prep=prep)
+        sage_ops.quant_k(k, ws, True, prep=prep)
+        sage_ops.quant_v(v, ws)
+        if e:
+            e[1].record()
+
+    run()
+    torch.cuda.synchronize()
+    for e in ev:
+        run(e)
+    torch.cuda.synchronize()
+    ms = sum(e[0].elapsed_time(e[1]) for e in ev) / iters
+    nbytes = 9.0 * w.elements
+    gbs = nbytes / (ms * 1e-3) / 1e9
+
+    def eager_norm_rope(x, weight):
+        """The same step as the model block runs it, with torch's own kernels on this GPU: RMSNorm in fp32
+        (ksana/operations/ops.py:62-72), then the rotation in complex128 (ksana/utils/rope.py:103-128)."""
+        B, L, H, D = x.shape
+        xf = x.reshape(B, L, H * D).float()
+        y = ((xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + 1e-6)) * weight).type_as(x).view(B, L, H, D)
+        f, h, wd = grid
+        parts = freqs.split([D // 2 - 2 * (D // 2 // 3), D // 2 // 3, D // 2 // 3], dim=1)
+        tab = torch.cat([parts[0][:f].view(f, 1, 1, -1).expand(f, h, wd, -1), parts[1][:h].view(1, h, 1, -1).expand(f, h, wd, -1),
+                         parts[2][:wd].view(1, 1, wd, -1).expand(f, h, wd, -1)], dim=-1).reshape(f * h * wd, 1, -1)
+        n = f * h * wd
+        z = torch.view_as_complex(y[0, :n].to(torch.float64).reshape(n, H, -1, 2))
+        z = torch.view_as_real(z * tab).flatten(2)
+        return torch.stack([torch.cat([z, y[0, n:]])]).type_as(x)
+
+    eager_norm_rope(q, wq)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    eager_norm_rope(q, wq)
+    eager_norm_rope(k, wk)
+    e1.record()
+    torch.cuda.synchronize()
+    eager_ms = e0.elapsed_time(e1)
+    return {
+        "what": "row statistic x2 + quantizer with RMSNorm(row of H*D) and 3-axis RoPE on q, k; V as before",
+        "grid": list(grid),
+        "ms": round(ms, 4),
+        "bound": "hbm",
+        "achieved": round(gbs, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(gbs / HBM_PEAK_GBS, 4),
+        "algorithmic_bytes": nbytes,
+        "eager_norm_rope_ms": round(eager_ms, 3),
+        "eager_note": "norm + rotation of q and k as the model block issues them (torch kernels on this GPU), to be added "
+                      "to quantizer_ms for the path without the on-the-fly step",
+    }
+
+
 def main() -> int:
     args = parse()
     if args.gpus != 1:
@@ -165,6 +245,9 @@ def main() -> int:
             "algorithmic_bytes": quant_bytes,
         },
     }
+    grid = WAN_GRIDS.get(w.name)
+    if grid is not None and w.B == 1:
+        rec["prep_quantizer"] = prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, max(3, args.steps // 2))
     if args.cpu_seconds > 0:
         rec["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
     print(json.dumps(rec))

@@ -40,6 +40,9 @@ struct PrepParams {
   const double* freqs;   // [rows, 64] complex128 as (re, im); nullptr = no rotation
   int L;
   int grid[kMaxPrepBatch][3];  // (frames, height, width) per batch entry
+  // Capacity (table rows) of the per-workgroup LDS copy of the rotation factors, filled in by the
+  // launcher for its kernel's rows per workgroup; lds_frames == 0: read `freqs` directly.
+  int lds_frames, lds_heights, lds_widths;
 };
 // inv_rms[b, l] from x[b, l, :H*128] (the row must be contiguous: sH == 128)
 hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps, float* inv_rms, hipStream_t s);

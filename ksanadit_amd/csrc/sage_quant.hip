@@ -70,8 +70,73 @@ __device__ __forceinline__ float through_half(float x) {
   return (float)(_Float16)x;
 }
 
+// Rotation factors for the rows of one workgroup, copied to LDS once.  The model's table is
+// [position on an axis][64 pairs] of complex128; a lane needs 8 of them (128 bytes) per row, four
+// times its payload, and fetched straight from the table those reads are 16 bytes out of 30-odd
+// different cache lines per load instruction - the L1 tag rate, not HBM, then sets the pace.  The
+// table is separable, so what a run of consecutive rows needs is small: the frames it touches
+// (22 pairs each), the image rows it touches (21 pairs each) and every column (21 pairs each).
+struct RopeLds {
+  const double2* frame;   // [frames touched][22], first = frame f0
+  const double2* height;  // [image rows touched][21], first = image row gr0 (counted across frames)
+  const double2* width;   // [grid width][21]
+  int f0, gr0;
+};
+
+constexpr int kRopeN0 = kRopeSplit0, kRopeN1 = kRopeSplit1 - kRopeSplit0, kRopeN2 = kD / 2 - kRopeSplit1;
+
+// All threads of the workgroup call this; rows [row0, row0 + nrows) of batch entry b are the
+// ones the workgroup will rotate.  Ends with a barrier.
+__device__ __forceinline__ RopeLds stage_rope(const PrepParams& pp, int b, int row0, int nrows, double2* lds) {
+  RopeLds rl;
+  rl.frame = lds;
+  rl.height = lds + pp.lds_frames * kRopeN0;
+  rl.width = rl.height + pp.lds_heights * kRopeN1;
+  const int gh = pp.grid[b][1], gw = pp.grid[b][2], plane = gh * gw;
+  const int r1 = min(row0 + nrows, pp.grid[b][0] * plane);  // exclusive; rows from here on are not rotated
+  rl.f0 = row0 / plane;
+  rl.gr0 = row0 / gw;
+  if (row0 < r1) {
+    const double2* tab = reinterpret_cast<const double2*>(pp.freqs);
+    const int nf = (r1 - 1) / plane - rl.f0 + 1, nh = (r1 - 1) / gw - rl.gr0 + 1;
+    const int t = threadIdx.x, nt = blockDim.x;
+    for (int idx = t; idx < nf * kRopeN0; idx += nt) {
+      const int r = idx / kRopeN0, i = idx - r * kRopeN0;
+      lds[idx] = tab[(int64_t)(rl.f0 + r) * (kD / 2) + i];
+    }
+    double2* hdst = lds + pp.lds_frames * kRopeN0;
+    for (int idx = t; idx < nh * kRopeN1; idx += nt) {
+      const int r = idx / kRopeN1, i = idx - r * kRopeN1;
+      hdst[idx] = tab[(int64_t)((rl.gr0 + r) % gh) * (kD / 2) + kRopeSplit0 + i];
+    }
+    double2* wdst = hdst + pp.lds_heights * kRopeN1;
+    for (int idx = t; idx < gw * kRopeN2; idx += nt) {
+      const int r = idx / kRopeN2, i = idx - r * kRopeN2;
+      wdst[idx] = tab[(int64_t)r * (kD / 2) + kRopeSplit1 + i];
+    }
+  }
+  __syncthreads();
+  return rl;
+}
+
+// n / d for 0 <= n < 2^24, 1 <= d: the fp32 quotient is off by at most one, fixed by the remainder test
+__device__ __forceinline__ int small_div(int n, int d, int* rem) {
+  int q = (int)(__int2float_rn(n) * __frcp_rn(__int2float_rn(d)));
+  int r = n - q * d;
+  if (r < 0) {
+    --q;
+    r += d;
+  } else if (r >= d) {
+    ++q;
+    r -= d;
+  }
+  *rem = r;
+  return q;
+}
+
 template <int DT>
-__device__ __forceinline__ void prep16(float* x, const PrepParams& pp, int b, int row, int h, int c16) {
+__device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const RopeLds& rl, int b, int row, int h,
+                                       int c16) {
   if (pp.inv_rms != nullptr) {
     const float r = pp.inv_rms[(int64_t)b * pp.L + row];
     const float4* w4 = reinterpret_cast<const float4*>(pp.weight + h * kD + c16 * 16);
@@ -88,21 +153,44 @@ __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, int b, in
     const int gh = pp.grid[b][1], gw = pp.grid[b][2];
     const int plane = gh * gw;
     if (row < pp.grid[b][0] * plane) {
-      const int f = row / plane, rem = row - f * plane;
-      const int hi = rem / gw, wi = rem - hi * gw;
+      int rem, wi;
+      const int f = small_div(row, plane, &rem);
+      const int hi = small_div(rem, gw, &wi);
+      // one table, three segments: the index is picked with integer selects so that every pair is a single
+      // load (selecting between three loads instead makes the compiler branch per pair)
+      auto rotate = [&](const double2* tab, int base_f, int base_h, int base_w) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int i = c16 * 8 + j;
-        const int tr = i < kRopeSplit0 ? f : (i < kRopeSplit1 ? hi : wi);
-        const double2 cs = *reinterpret_cast<const double2*>(pp.freqs + ((int64_t)tr * (kD / 2) + i) * 2);
-        const double a = (double)x[2 * j], bb = (double)x[2 * j + 1];
-        const double re = a * cs.x - bb * cs.y;
-        const double im = a * cs.y + bb * cs.x;
-        x[2 * j] = through_half<DT>((float)re);
-        x[2 * j + 1] = through_half<DT>((float)im);
-      }
+        for (int j = 0; j < 8; ++j) {
+          const int i = c16 * 8 + j;
+          const int idx = (i < kRopeSplit0 ? base_f : (i < kRopeSplit1 ? base_h : base_w)) + i;
+          const double2 cs = tab[idx];
+          const double a = (double)x[2 * j], bb = (double)x[2 * j + 1];
+          const double re = a * cs.x - bb * cs.y;
+          const double im = a * cs.y + bb * cs.x;
+          x[2 * j] = through_half<DT>((float)re);
+          x[2 * j + 1] = through_half<DT>((float)im);
+        }
+      };
+      if (pp.lds_frames > 0)  // uniform
+        rotate(rl.frame, (f - rl.f0) * kRopeN0,
+               (int)(rl.height - rl.frame) + (f * gh + hi - rl.gr0) * kRopeN1 - kRopeSplit0,
+               (int)(rl.width - rl.frame) + wi * kRopeN2 - kRopeSplit1);
+      else
+        rotate(reinterpret_cast<const double2*>(pp.freqs), f * (kD / 2), hi * (kD / 2), wi * (kD / 2));
     }
   }
+}
+
+// Dynamic LDS of the kernels that rotate: the staged factors.
+extern __shared__ __attribute__((aligned(16))) double2 s_rope_tables[];
+
+template <bool PRE>
+__device__ __forceinline__ RopeLds maybe_stage_rope(const PrepParams& pp, int b, int row0, int nrows) {
+  RopeLds rl{};
+  if constexpr (PRE) {
+    if (pp.freqs != nullptr && pp.lds_frames > 0) rl = stage_rope(pp, b, row0, nrows, s_rope_tables);
+  }
+  return rl;
 }
 
 // 1 / sqrt(mean(x^2) + eps) of every token row x[b, l, 0 : n8*8].  One wave per row: lane i takes the
@@ -143,13 +231,14 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
   const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const uint16_t* base = x + b * sB + h * sH + c16 * 16;
+  const RopeLds rl = maybe_stage_rope<PRE>(pp, b, ch * kMeanChunk, kMeanChunk);
   float rows[kMeanChunk / kSlots][16];
 #pragma unroll
   for (int i = 0; i < kMeanChunk / kSlots; ++i) {
     const int row = ch * kMeanChunk + i * kSlots + slot;
     load_row16<DT>(base + (int64_t)row * sL, row < L, rows[i]);
     if constexpr (PRE) {
-      if (row < L) prep16<DT>(rows[i], pp, b, row, h, c16);
+      if (row < L) prep16<DT>(rows[i], pp, rl, b, row, h, c16);
     }
   }
   float acc[16];
@@ -237,6 +326,32 @@ __global__ __launch_bounds__(kFinThreads) void v_scale_finalize_kernel(const flo
   }
 }
 
+// Value of lane (id ^ M) for M = 1, 2, 4, through DPP (the exchange then rides on the consuming
+// VALU instruction instead of a round trip through the LDS crossbar).
+//   quad_perm [1,0,3,2] = id ^ 1;  quad_perm [2,3,0,1] = id ^ 2;
+//   row_half_mirror (id -> 7 - id within 8 lanes) followed by quad_perm [3,2,1,0] (id ^ 3) = id ^ 4.
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+  static_assert(M == 1 || M == 2 || M == 4, "only within groups of 8 lanes");
+  const int iv = __float_as_int(v);
+  if constexpr (M == 1) return __int_as_float(__builtin_amdgcn_mov_dpp(iv, 0xB1, 0xF, 0xF, true));
+  if constexpr (M == 2) return __int_as_float(__builtin_amdgcn_mov_dpp(iv, 0x4E, 0xF, 0xF, true));
+  const int t = __builtin_amdgcn_mov_dpp(iv, 0x141, 0xF, 0xF, true);
+  return __int_as_float(__builtin_amdgcn_mov_dpp(t, 0x1B, 0xF, 0xF, true));
+}
+
+template <int M>
+__device__ __forceinline__ void fwht_cross_stage(float* x, int c16) {
+  // the lane holding the "b" half of a pair computes a - b as (+a) + (-b)
+  const unsigned flip = (c16 & M) ? 0x80000000u : 0u;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const float other = lane_xor<M>(x[e]);
+    const float own = __uint_as_float(__float_as_uint(x[e]) ^ flip);
+    x[e] = other + own;
+  }
+}
+
 // Unnormalised Walsh-Hadamard transform of one 128-channel row held by 8 adjacent lanes x 16
 // values (channel = 16*c16 + e).  Butterflies (a, b) -> (a + b, a - b) with stride 1, 2, 4, 8
 // inside the lane, then 16, 32, 64 across lanes c16 ^ 1, ^ 2, ^ 4 - in exactly that order.
@@ -252,16 +367,9 @@ __device__ __forceinline__ void fwht128(float* x, int c16) {
       }
     }
   }
-#pragma unroll
-  for (int m = 1; m <= 4; m <<= 1) {
-    const bool upper = (c16 & m) != 0;  // this lane holds the "b" half of the pair
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const float other = __shfl_xor(x[e], m);
-      const float own = upper ? -x[e] : x[e];
-      x[e] = other + own;
-    }
-  }
+  fwht_cross_stage<1>(x, c16);
+  fwht_cross_stage<2>(x, c16);
+  fwht_cross_stage<4>(x, c16);
 }
 
 // max over the workgroup of a non-negative per-thread value
@@ -305,13 +413,14 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
   const uint16_t* base = q + b * sB + h * sH + c16 * 16;
   constexpr int kRowsPerWg = 128, R = kRowsPerWg / kSlots;
   const int64_t bh = (int64_t)b * H + h;
+  const RopeLds rl = maybe_stage_rope<PRE>(pp, b, blk * kRowsPerWg, kRowsPerWg);
   float x[R][16];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = blk * kRowsPerWg + i * kSlots + slot;
     load_row16<DT>(base + (int64_t)row * sL, row < L, x[i]);
     if constexpr (PRE) {
-      if (row < L) prep16<DT>(x[i], pp, b, row, h, c16);
+      if (row < L) prep16<DT>(x[i], pp, rl, b, row, h, c16);
     }
   }
 #pragma unroll
@@ -324,8 +433,9 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
       x[i][e] = x[i][e] * premul;
       amax = fmaxf(amax, fabsf(x[i][e]));
     }
-#pragma unroll
-    for (int m = 1; m <= 4; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
+    amax = fmaxf(amax, lane_xor<1>(amax));
+    amax = fmaxf(amax, lane_xor<2>(amax));
+    amax = fmaxf(amax, lane_xor<4>(amax));
     const bool nz = amax > 0.0f;
     const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
     if (c16 == 0) q_scale[bh * lq_pad + row] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
@@ -353,6 +463,7 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
 #pragma unroll
   for (int e = 0; e < 16; ++e) km[e] = k_mean[bh * kD + c16 * 16 + e];
   constexpr int R = kBlkK / kSlots;
+  const RopeLds rl = maybe_stage_rope<PRE>(pp, b, blk * kBlkK, kBlkK);
   float x[R][16];
   float amax = 0.0f;
 #pragma unroll
@@ -361,7 +472,7 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
     const bool valid = row < L;
     load_row16<DT>(base + (int64_t)row * sL, valid, x[i]);
     if constexpr (PRE) {
-      if (valid) prep16<DT>(x[i], pp, b, row, h, c16);
+      if (valid) prep16<DT>(x[i], pp, rl, b, row, h, c16);
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -459,6 +570,24 @@ __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __res
     }                                            \
   } while (0)
 
+// Sizes the LDS copy of the rotation factors for kernels that give `rows_per_wg` consecutive rows to
+// a workgroup; returns the dynamic LDS bytes (0: the kernel reads the table directly).
+static size_t plan_rope_lds(PrepParams* pp, int B, int rows_per_wg) {
+  pp->lds_frames = pp->lds_heights = pp->lds_widths = 0;
+  if (pp->freqs == nullptr) return 0;
+  int nf = 0, nh = 0, nw = 0;
+  for (int b = 0; b < B; ++b) {
+    const int gh = pp->grid[b][1], gw = pp->grid[b][2];
+    nf = max(nf, (rows_per_wg - 1) / (gh * gw) + 2);
+    nh = max(nh, (rows_per_wg - 1) / gw + 2);
+    nw = max(nw, gw);
+  }
+  const size_t bytes = ((size_t)nf * kRopeN0 + (size_t)nh * kRopeN1 + (size_t)nw * kRopeN2) * sizeof(double2);
+  if (bytes > 48 * 1024) return 0;  // unusual grids (very wide, or planes of a few tokens): direct reads
+  pp->lds_frames = nf, pp->lds_heights = nh, pp->lds_widths = nw;
+  return bytes;
+}
+
 hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps, float* inv_rms, hipStream_t s) {
   const dim3 grid((L + 3) / 4, B), block(kThreads);
   KSANA_DISPATCH_DT(x.dtype, (row_inv_rms_kernel<DT><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, L, H * kD / 8,
@@ -475,8 +604,11 @@ hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, fl
       col_partial_kernel<DT, 1, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none);
     else if (prep == nullptr)
       col_partial_kernel<DT, 0, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none);
-    else
-      col_partial_kernel<DT, 0, true><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, *prep);
+    else {
+      PrepParams pp = *prep;
+      const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
+      col_partial_kernel<DT, 0, true><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, pp);
+    }
   });
   return hipGetLastError();
 }
@@ -500,9 +632,12 @@ hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, fl
     if (prep == nullptr)
       quant_q_kernel<DT, false><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
                                                         none);
-    else
-      quant_q_kernel<DT, true><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
-                                                       *prep);
+    else {
+      PrepParams pp = *prep;
+      const size_t lds = plan_rope_lds(&pp, B, 128);
+      quant_q_kernel<DT, true><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
+                                                         pp);
+    }
   });
   return hipGetLastError();
 }
@@ -515,9 +650,12 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
     if (prep == nullptr)
       quant_k_kernel<DT, false><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
                                                         none);
-    else
-      quant_k_kernel<DT, true><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
-                                                       *prep);
+    else {
+      PrepParams pp = *prep;
+      const size_t lds = plan_rope_lds(&pp, B, kBlkK);
+      quant_k_kernel<DT, true><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
+                                                         pp);
+    }
   });
   return hipGetLastError();
 }
