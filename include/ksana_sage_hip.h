@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 4
+#define KSANA_SAGE_ABI_VERSION 5
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -150,6 +150,19 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], con
 int ksana_sage_attn_fwd(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
                         const ksana_sage_shape* shape, const int32_t* k_lens, int causal, int flags, void* stream);
 
+/* ksana_sage_attn_fwd restricted by a block mask: block_mask is a device array of int8
+ * [B, Hq, ceil(Lq/128), ceil(Lk/64)]; a non-zero entry lets the 128 query rows of its row attend to
+ * the 64 keys of its column, zero hides them; dense inside a block.  mask_strides are the element
+ * strides of the two leading dimensions (0 broadcasts over batch / heads); the last two dimensions
+ * are contiguous.  Query rows whose mask row is all zero come out as zeros.  Lk <= 131072.
+ * Replaces block_sparse_sage2_attn_cuda(q, k, v, mask_id=..., tensor_layout="NHD")
+ * (radial_sage_attn.py:24,170-176: the same mask shape and block sizes); block_mask == NULL is
+ * ksana_sage_attn_fwd.  Key tiles neither 128-row half of a 256-row workgroup asks for are skipped. */
+int ksana_sage_attn_fwd_masked(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
+                               const ksana_sage_shape* shape, const int8_t* block_mask,
+                               const int64_t mask_strides[2], const int32_t* k_lens, int causal, int flags,
+                               void* stream);
+
 /* The whole path in one call: quant_q, quant_k, quant_v, attn_fwd on `stream`.
  * Replaces sageattn(q, k, v, tensor_layout="NHD", is_causal=causal) (sage_attn.py:75-81). */
 int ksana_sage_forward(const void* q, const void* k, const void* v, void* o, int dtype,
@@ -164,6 +177,13 @@ int ksana_sage_forward_prep(const void* q, const void* k, const void* v, void* o
                             const int64_t o_strides[4], const ksana_sage_shape* shape, const ksana_sage_prep* prep,
                             const int32_t* k_lens, float sm_scale, int smooth_k, int causal, int flags,
                             void* workspace, void* stream);
+
+/* ksana_sage_forward with the block mask of ksana_sage_attn_fwd_masked. */
+int ksana_sage_forward_masked(const void* q, const void* k, const void* v, void* o, int dtype,
+                              const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                              const int64_t o_strides[4], const ksana_sage_shape* shape, const int8_t* block_mask,
+                              const int64_t mask_strides[2], const int32_t* k_lens, float sm_scale, int smooth_k,
+                              int causal, int flags, void* workspace, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -29,6 +29,8 @@ EXPORTS = (
     "ksana_sage_quant_q_prep",
     "ksana_sage_quant_k_prep",
     "ksana_sage_forward_prep",
+    "ksana_sage_attn_fwd_masked",
+    "ksana_sage_forward_masked",
 )
 
 
@@ -85,6 +87,11 @@ def _declare(lib):
     lib.ksana_sage_quant_k_prep.argtypes, lib.ksana_sage_quant_k_prep.restype = [vp, i, st, sp, pp, i, vp, vp], i
     lib.ksana_sage_forward_prep.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, pp, vp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward_prep.restype = i
+    ms = C.POINTER(C.c_int64)
+    lib.ksana_sage_attn_fwd_masked.argtypes = [vp, vp, i, st, sp, vp, ms, vp, i, i, vp]
+    lib.ksana_sage_attn_fwd_masked.restype = i
+    lib.ksana_sage_forward_masked.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, ms, vp, f, i, i, i, vp, vp]
+    lib.ksana_sage_forward_masked.restype = i
 
 
 def library_present() -> bool:

@@ -99,7 +99,7 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
   }
 }
 
-template <int DT, bool kPwlExp>
+template <int DT, bool kPwlExp, bool kSparse>
 __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg, int n_wg,
                                                                      int wg_per_xcd) {
   // Consecutive workgroup ids land on consecutive XCDs (8 per chip, one L2 each).  Give every
@@ -121,13 +121,16 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   // keys [0, lk) of this batch take part: all of them, or the caller's per-batch count
   int lk = p.Lk;
   if (p.k_lens != nullptr) lk = min(max(p.k_lens[b], 0), p.Lk);  // uniform: a scalar load
-  if (lk == 0) {  // softmax over no key: the output rows are defined as zeros
+  auto write_zero_rows = [&]() {  // softmax over no key: the output rows are defined as zeros
     const int q = q0 + l32;
     if (q < p.Lq) {
       uint4* orow = reinterpret_cast<uint4*>(p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH + 64 * hh);
 #pragma unroll
       for (int i = 0; i < 8; ++i) orow[i] = make_uint4(0, 0, 0, 0);
     }
+  };
+  if (lk == 0) {
+    write_zero_rows();
     return;
   }
 
@@ -178,18 +181,67 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   // K scales live in LDS behind the ring: a per-tile global load would share the in-order
   // vmcnt queue with the tile copies and stall on all of them
   float* s_ks = reinterpret_cast<float*>(smem + kStages * kStageBytes);
-  for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
+
+  // ---- block mask: the workgroup's list of key tiles ---------------------------------------
+  // A mask row covers 128 query rows, a workgroup two of them (waves 0-3, waves 4-7).  Wave 0
+  // compacts, in key order, the tiles either row asks for into LDS: entry = tile | row-0 flag
+  // << 16 | row-1 flag << 17.  The loop below then walks list positions instead of tile
+  // numbers; a wave whose row does not ask for a tile zeroes its probabilities for it and
+  // leaves its running maximum alone, so the result is exactly the masked softmax.
+  int* s_list = reinterpret_cast<int*>(smem + kStages * kStageBytes + kSparseMaxKeyTiles * 4);
+  int n_tiles = nkb;  // loop length: list entries with a mask, key tiles without
+  if constexpr (kSparse) {
+    if (wave == 0) {
+      const int nqm = (p.Lq + kMaskBlkQ - 1) / kMaskBlkQ;
+      const int8_t* m0 = p.block_mask + b * p.mask_sB + h * p.mask_sH + (int64_t)(2 * qwg) * p.nkb;
+      const bool two = 2 * qwg + 1 < nqm;
+      int base = 0;
+      for (int j0 = 0; j0 < nkb; j0 += 64) {
+        const int j = j0 + lane;
+        int f0 = 0, f1 = 0;
+        if (j < nkb) {
+          f0 = m0[j] != 0;
+          f1 = two && m0[p.nkb + j] != 0;
+        }
+        const bool keep = (f0 | f1) != 0;
+        const unsigned long long bal = __ballot(keep);
+        const int pre = __builtin_amdgcn_mbcnt_hi((unsigned)(bal >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)bal, 0));
+        if (keep) s_list[base + pre] = j | (f0 << 16) | (f1 << 17);
+        base += __popcll(bal);
+      }
+      if (lane == 0) s_list[kSparseMaxKeyTiles] = base;
+    }
+    __syncthreads();
+    n_tiles = __builtin_amdgcn_readfirstlane(s_list[kSparseMaxKeyTiles]);
+    if (n_tiles == 0) {  // neither mask row allows any key
+      write_zero_rows();
+      return;
+    }
+    for (int i = tid; i < n_tiles; i += kThreadsAttn) s_ks[i] = ks_ptr[s_list[i] & 0xffff];
+  } else {
+    for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
+  }
+  // key tile behind loop position jj, and whether this wave's mask row asks for it
+  auto tile_of = [&](int jj) -> int {
+    if constexpr (kSparse) return __builtin_amdgcn_readfirstlane(s_list[jj]) & 0xffff;
+    return jj;
+  };
+  auto mine_at = [&](int jj) -> bool {
+    if constexpr (kSparse) return ((__builtin_amdgcn_readfirstlane(s_list[jj]) >> (16 + (wave >> 2))) & 1) != 0;
+    return true;
+  };
 
   // ---- asynchronous tile copies: HBM/L2 -> LDS without passing through registers ----------
   // Each wave moves its 1 KiB slice of the K tile and of the V^T tile (lane i -> byte 16*i of
   // the slice).  Copies retire in issue order, so "at most 2*n outstanding" == "all but the
   // newest n tiles have landed".
-  const bool has_tail = (lk & (kBlkK - 1)) != 0;  // keys >= lk live only in the last tile
-  const int n_main = has_tail ? nkb - 1 : nkb;       // tiles handled by the pipelined loop
+  // keys >= lk live only in the last key tile, which (if the list holds it) is the last entry
+  const bool has_tail = (lk & (kBlkK - 1)) != 0 && tile_of(n_tiles - 1) == nkb - 1;
+  const int n_main = has_tail ? n_tiles - 1 : n_tiles;  // entries handled by the pipelined loop
   auto issue_copy = [&](int tile) {
     // clamped: past the end the last tile is copied again into a stage nobody reads any more,
     // which keeps the loop free of branches and the outstanding-copy count constant
-    const int jl = min(tile, nkb - 1);
+    const int jl = tile_of(min(tile, n_tiles - 1));
     const uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes + wave * 1024;
     lds_copy16(k_src + (int64_t)jl * kTileBytes, copy_off, dst);
     lds_copy16(v_src + (int64_t)jl * kTileBytes, copy_off, dst + kTileBytes);
@@ -316,14 +368,17 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     kf[0] = k_frag(0);
     kf[1] = k_frag(1);
     kf[2] = k_frag(2);
-    const float ks_nxt = s_ks[min(j + 1, nkb - 1)];
+    const float ks_nxt = s_ks[min(j + 1, n_tiles - 1)];
+    const bool mine = mine_at(j);
     issue_copy(j + kAhead);
     if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
     // row sums of tile j-1: 64 matrix cycles that run under the max finalisation below
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
     const float sc = qs * ks_cur;
     const float mneg = -kMagicF * sc;
-    alpha_prev = update_max(mx_cur, sc, mneg);
+    // a tile this wave's mask row does not ask for leaves the running maximum alone (wave-uniform
+    // branch); its probabilities are zeroed where they are packed
+    alpha_prev = mine ? update_max(mx_cur, sc, mneg) : 1.0f;
     // exponent of key r: x = sc*dot - m_run + shift, with the magic folded into the constant
     // (which is therefore off by at most ~1.5 integer steps of the dot product)
     const float c = (kPShift - m_run) + mneg;
@@ -375,6 +430,11 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     }
     mx_cur = max(max(pm[0], pm[1]), max(pm[2], pm[3]));
     ks_cur = ks_nxt;
+    if constexpr (kSparse) {
+      const int keep = mine ? -1 : 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pf[i] &= keep;
+    }
     pf_prev = pf;
     // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
     tile_barrier();
@@ -396,8 +456,8 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_prev);
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
   }
-  if (has_tail) {  // ragged last tile, not pipelined: mask keys >= lk
-    const int j = nkb - 1;
+  if (has_tail && mine_at(n_tiles - 1)) {  // ragged last tile, not pipelined: mask keys >= lk
+    const int j = nkb - 1, jj = n_tiles - 1;
     v16i (&s_cur)[2] = (n_main & 1) ? s_b : s_a;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -406,7 +466,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         const int key = j * kBlkK + 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
         if (key >= lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
       }
-    const float sc = qs * s_ks[j];
+    const float sc = qs * s_ks[jj];
     const float mneg = -kMagicF * sc;
     scale_o(update_max(lane_max(s_cur), sc, mneg));
     const float c = (kPShift - m_run) + mneg;
@@ -427,14 +487,15 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         }
         pf[4 * t + g] = w & (int)keep;
       }
-    const uint8_t* vst = smem + (j & (kStages - 1)) * kStageBytes + kTileBytes;
+    const uint8_t* vst = smem + (jj & (kStages - 1)) * kStageBytes + kTileBytes;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf);
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, lacc, 0, 0, 0, 0, 0, 0);
   }
 
   // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
-  const float inv_l = 1.0f / lacc[0];
+  // a mask row that allows none of its keys has an empty sum: its rows are zeros, not 0/0
+  const float inv_l = (!kSparse || lacc[0] > 0.0f) ? 1.0f / lacc[0] : 0.0f;
   const int q = q0 + l32;
   if (q < p.Lq) {
     uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
@@ -452,7 +513,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   }
 }
 
-template <int DT, bool kPwlExp>
+template <int DT, bool kPwlExp, bool kSparse>
 hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
   // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
@@ -463,12 +524,14 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   if (!requested[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStageBytes + kMaxKeyTiles * 4);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kSparse ? kStages * kStageBytes + 2 * kSparseMaxKeyTiles * 4 + 1024
+                                    : kStages * kStageBytes + kMaxKeyTiles * 4);
     if (e != hipSuccess) return e;
     requested[dev].store(true, std::memory_order_release);
   }
-  sage_attn_fwd_kernel<DT, kPwlExp><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  sage_attn_fwd_kernel<DT, kPwlExp, kSparse><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
 }
 
@@ -480,14 +543,24 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const int n_wg = p.B * p.Hq * n_qwg;
   const int wg_per_xcd = (n_wg + 7) / 8;
   const dim3 grid(wg_per_xcd * 8), block(kThreadsAttn);
+  const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
+  if (p.block_mask != nullptr) {
+    if (p.nkb > kSparseMaxKeyTiles) return hipErrorInvalidValue;
+    // tile ring + K scales of the listed tiles + the tile list and its length
+    const size_t lds = kStages * kStageBytes + 2 * kSparseMaxKeyTiles * 4 + 1024;
+    if (p.exact_exp2)
+      return bf16 ? launch_variant<KSANA_SAGE_BF16, false, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
+                  : launch_variant<KSANA_SAGE_FP16, false, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, true, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, true, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
+  }
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
   const size_t lds = kStages * kStageBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
-  const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
   if (p.exact_exp2)
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
-  return bf16 ? launch_variant<KSANA_SAGE_BF16, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
-              : launch_variant<KSANA_SAGE_FP16, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
+  return bf16 ? launch_variant<KSANA_SAGE_BF16, true, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
+              : launch_variant<KSANA_SAGE_FP16, true, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
 }
 
 }  // namespace ksana_sage

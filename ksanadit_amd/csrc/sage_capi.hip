@@ -74,6 +74,21 @@ int check_ws(const void* ws) {
   return 0;
 }
 
+int check_mask(const ksana_sage_shape* s, const int8_t* block_mask, const int64_t mask_st[2]) {
+  if (!block_mask) return 0;
+  if (!mask_st) return fail(KSANA_SAGE_EINVAL, "block_mask given without mask_strides");
+  if (mask_st[0] < 0 || mask_st[1] < 0) return fail(KSANA_SAGE_EINVAL, "negative mask stride");
+  if (s->Lk > ksana_sage::kSparseMaxKeyTiles * ksana_sage::kBlkK)
+    return fail(KSANA_SAGE_ENOTSUP, "Lk=%d exceeds %d with a block mask (the tile list is kept in LDS)", s->Lk,
+                ksana_sage::kSparseMaxKeyTiles * ksana_sage::kBlkK);
+  return 0;
+}
+
+int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
+                 const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4], const ksana_sage_shape* s,
+                 const ksana_sage_prep* prep, const int8_t* block_mask, const int64_t mask_st[2],
+                 const int32_t* k_lens, float sm_scale, int smooth_k, int causal, int flags, void* ws, void* stream);
+
 // Validates `prep` for one tensor (`weight` is that tensor's norm weight) and fills the kernel-side
 // parameters.  *out stays nullptr when there is nothing to apply.
 int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name, const int64_t st[4], int B, int L,
@@ -249,7 +264,14 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksan
 
 int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
                         const int32_t* k_lens, int causal, int flags, void* stream) {
+  return ksana_sage_attn_fwd_masked(ws, o, dtype, o_st, s, nullptr, nullptr, k_lens, causal, flags, stream);
+}
+
+int ksana_sage_attn_fwd_masked(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
+                               const int8_t* block_mask, const int64_t mask_st[2], const int32_t* k_lens, int causal,
+                               int flags, void* stream) {
   if (int rc = check_shape(s)) return rc;
+  if (int rc = check_mask(s, block_mask, mask_st)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
   if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
@@ -269,6 +291,9 @@ int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;
   p.exact_exp2 = (flags & KSANA_SAGE_FLAG_PWL_EXP2) ? 0 : 1;
   p.k_lens = k_lens;
+  p.block_mask = block_mask;
+  p.mask_sB = block_mask ? mask_st[0] : 0;
+  p.mask_sH = block_mask ? mask_st[1] : 0;
   hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
 }
@@ -285,7 +310,28 @@ int ksana_sage_forward_prep(const void* q, const void* k, const void* v, void* o
                             const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
                             const ksana_sage_shape* s, const ksana_sage_prep* prep, const int32_t* k_lens,
                             float sm_scale, int smooth_k, int causal, int flags, void* ws, void* stream) {
+  return forward_impl(q, k, v, o, dtype, q_st, k_st, v_st, o_st, s, prep, nullptr, nullptr, k_lens, sm_scale, smooth_k,
+                      causal, flags, ws, stream);
+}
+
+int ksana_sage_forward_masked(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
+                              const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4],
+                              const ksana_sage_shape* s, const int8_t* block_mask, const int64_t mask_st[2],
+                              const int32_t* k_lens, float sm_scale, int smooth_k, int causal, int flags, void* ws,
+                              void* stream) {
+  return forward_impl(q, k, v, o, dtype, q_st, k_st, v_st, o_st, s, nullptr, block_mask, mask_st, k_lens, sm_scale,
+                      smooth_k, causal, flags, ws, stream);
+}
+
+}  // extern "C"
+
+namespace {
+int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
+                 const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4], const ksana_sage_shape* s,
+                 const ksana_sage_prep* prep, const int8_t* block_mask, const int64_t mask_st[2],
+                 const int32_t* k_lens, float sm_scale, int smooth_k, int causal, int flags, void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
+  if (int rc = check_mask(s, block_mask, mask_st)) return rc;
   if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
   // validate everything before the first launch so a bad argument leaves no partial work
   if (int rc = check_tensor("q", q, dtype, q_st, s->B, s->Lq, s->Hq)) return rc;
@@ -307,7 +353,6 @@ int ksana_sage_forward_prep(const void* q, const void* k, const void* v, void* o
   if (int rc = ksana_sage_quant_q_prep(q, dtype, q_st, s, prep, sm_scale, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_k_prep(k, dtype, k_st, s, prep, smooth_k, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_v(v, dtype, v_st, s, ws, stream)) return rc;
-  return ksana_sage_attn_fwd(ws, o, dtype, o_st, s, k_lens, causal, flags, stream);
+  return ksana_sage_attn_fwd_masked(ws, o, dtype, o_st, s, block_mask, mask_st, k_lens, causal, flags, stream);
 }
-
-}  // extern "C"
+}  // namespace

@@ -71,7 +71,13 @@ struct AttnParams {
   int B, Hq, Hkv, Lq, Lk, lq_pad, nkb;
   int exact_exp2;  // 1: exp2 on the transcendental unit; 0: piecewise-linear e4m3 code (faster)
   const int32_t* k_lens;  // optional [B]: batch b attends to keys [0, clamp(k_lens[b], 0, Lk)); nullptr = all
+  // optional block mask, int8 [B, Hq, ceil(Lq/128), ceil(Lk/64)] (rows contiguous): non-zero = the 128 query
+  // rows attend to the 64 keys; nullptr = dense
+  const int8_t* block_mask;
+  int64_t mask_sB, mask_sH;  // element strides of the two leading dims (0 broadcasts)
 };
+constexpr int kMaskBlkQ = 128;           // query rows per mask row (two per workgroup)
+constexpr int kSparseMaxKeyTiles = 2048; // key tiles per head with a block mask (tile list lives in LDS)
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s);
 
 }  // namespace ksana_sage

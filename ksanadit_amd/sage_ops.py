@@ -229,17 +229,45 @@ def _k_lens_arg(k_lens, batch: int, device: torch.device):
     return k_lens.to(device=device, dtype=torch.int32).contiguous()
 
 
+MASK_BLKQ, MASK_BLKK = 128, 64  # query rows / keys per block-mask entry
+
+
+def _block_mask_arg(block_mask, B: int, H: int, Lq: int, Lk: int, device):
+    """``block_mask`` as the int8 device array the library reads, plus its two leading strides.
+    Accepts ``[nq, nk]``, ``[H, nq, nk]`` or ``[B, H, nq, nk]`` (size-1 or expanded leading dims broadcast)."""
+    if block_mask is None:
+        return None, None
+    m = torch.as_tensor(block_mask)
+    nq, nk = -(-Lq // MASK_BLKQ), -(-Lk // MASK_BLKK)
+    while m.dim() < 4:
+        m = m.unsqueeze(0)
+    if m.dim() != 4 or m.shape[2:] != (nq, nk) or m.shape[0] not in (1, B) or m.shape[1] not in (1, H):
+        raise ValueError(f"block_mask must be [.., {nq}, {nk}] with leading dims (1|{B}, 1|{H}), got {tuple(m.shape)}")
+    lead_b = 1 if (m.shape[0] == 1 or m.stride(0) == 0) else B
+    lead_h = 1 if (m.shape[1] == 1 or m.stride(1) == 0) else H
+    m = m[:lead_b, :lead_h].to(device=device, dtype=torch.int8).contiguous()
+    strides = (C.c_int64 * 2)(m.stride(0) if lead_b > 1 else 0, m.stride(1) if lead_h > 1 else 0)
+    return m, strides
+
+
 def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False,
-             k_lens=None) -> torch.Tensor:
+             k_lens=None, block_mask=None) -> torch.Tensor:
     """Attention on the quantized operands in ``ws``.  ``k_lens`` (optional, one int per batch entry): batch ``b``
     attends to keys ``[0, k_lens[b])`` only, the meaning the reference's callers give it (wan_model.py:182-189,
-    flash_attn.py:131-139); a batch entry without keys yields zeros."""
+    flash_attn.py:131-139); a batch entry without keys yields zeros.  ``block_mask`` (optional, int8/bool
+    ``[B, H, ceil(Lq/128), ceil(Lk/64)]``, leading dims may broadcast): block ``(i, j)`` non-zero lets query rows
+    ``128 i ..`` attend to keys ``64 j ..`` - the ``mask_id`` of the reference's block-sparse call
+    (radial_sage_attn.py:170-176)."""
     _require_hip(out)
     lib = _capi.load()
     flags = _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0
     kl = _k_lens_arg(k_lens, out.shape[0], out.device)
-    rc = lib.ksana_sage_attn_fwd(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
-                                 None if kl is None else kl.data_ptr(), int(causal), flags, _stream_ptr(out.device))
+    s = ws.shape
+    mask, mask_st = _block_mask_arg(block_mask, s.B, s.Hq, s.Lq, s.Lk, out.device)
+    rc = lib.ksana_sage_attn_fwd_masked(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
+                                        None if mask is None else mask.data_ptr(), mask_st,
+                                        None if kl is None else kl.data_ptr(), int(causal), flags,
+                                        _stream_ptr(out.device))
     _capi.check(rc, "ksana_sage_attn_fwd")
     return out
 
@@ -256,12 +284,14 @@ def sageattn(
     pwl_exp2: bool = False,
     k_lens=None,
     prep: WanPrep | None = None,
+    block_mask=None,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
 
     ``k_lens`` (optional, one int per batch entry) limits batch ``b`` to its first ``k_lens[b]`` keys.
     ``prep`` (optional, "NHD" only): q and k are the raw projections and the block's RMSNorm + RoPE are applied
     while they are read (see ``WanPrep``).
+    ``block_mask`` (optional): block-sparse attention, see ``attn_fwd`` (not together with ``prep``).
 
     ``pwl_exp2=True`` computes the e4m3 code of every probability directly (exp2 with a
     piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate."""
@@ -286,6 +316,18 @@ def sageattn(
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)
+    if block_mask is not None:
+        if prep is not None:
+            raise ValueError("block_mask and prep cannot be combined in one call; quantize with prep, then attn_fwd")
+        mask, mask_st = _block_mask_arg(block_mask, B, Hq, Lq, k.shape[1], q.device)
+        rc = lib.ksana_sage_forward_masked(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
+            _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape), mask.data_ptr(), mask_st,
+            None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal),
+            _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
+        )
+        _capi.check(rc, "ksana_sage_forward_masked")
+        return out.transpose(1, 2) if tensor_layout == "HND" else out
     c_prep, _keep = (None, None) if prep is None else prep.to_c(q.device)
     rc = lib.ksana_sage_forward_prep(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
@@ -303,3 +345,11 @@ def wan_self_attention(q_proj: torch.Tensor, k_proj: torch.Tensor, v_proj: torch
     The normed and rotated q and k are never written to memory."""
     q, k, v = (_as_heads(t, num_heads) for t in (q_proj, k_proj, v_proj))
     return sageattn(q, k, v, tensor_layout="NHD", prep=prep, **kwargs)
+
+
+def block_sparse_sage2_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask_id: torch.Tensor,
+                            tensor_layout: str = "NHD", **kwargs) -> torch.Tensor:
+    """Same call shape as the reference's ``block_sparse_sage2_attn_cuda(q, k, v, mask_id=..., tensor_layout="NHD")``
+    (ksana/operations/attention/backends/radial_sage_attn/radial_sage_attn.py:24,170-176): ``mask_id`` is
+    ``[B, H, ceil(Lq/128), ceil(Lk/64)]``, non-zero = attend."""
+    return sageattn(q, k, v, tensor_layout=tensor_layout, block_mask=mask_id, **kwargs)

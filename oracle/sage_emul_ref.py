@@ -42,13 +42,15 @@ def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
 
 
 def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True,
-                         exact_exp2=True, k_lens=None):
+                         exact_exp2=True, k_lens=None, block_mask=None):
     """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
 
     ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
     decides where each P lands on the e4m3 grid, so the fp8 rounding of P matches the kernel's
     (a full softmax rounds P relative to the FINAL max - same accuracy, different bits).
     ``k_lens``: batch ``b`` uses keys ``[0, k_lens[b])`` of the quantized operands (online form only).
+    ``block_mask`` (``[B|1, H|1, ceil(Lq/128), ceil(Lk/64)]``): query rows ``128 i ..`` walk only the key tiles ``j``
+    with a non-zero entry ``(i, j)``; rows without any tile give zeros (online form only).
     """
     B, H, Lq, D = q_i8.shape
     Hkv, Lk = k_i8.shape[1], k_i8.shape[2]
@@ -56,8 +58,13 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     out = torch.empty(B, Lq, H, D, dtype=out_dtype)
     qs_row = q_scale.repeat_interleave(BLKQ, dim=2)[:, :, :Lq]  # [B, H, Lq] (BLKQ == 1: already per row)
     ks_col = k_scale.repeat_interleave(BLKK, dim=2)[:, :, :Lk]  # [B, Hkv, Lk]
-    if k_lens is not None and not online:
-        raise NotImplementedError("k_lens with the full-softmax form")
+    if (k_lens is not None or block_mask is not None) and not online:
+        raise NotImplementedError("k_lens / block_mask with the full-softmax form")
+    if block_mask is not None:
+        bm = torch.as_tensor(block_mask) != 0
+        while bm.dim() < 4:
+            bm = bm.unsqueeze(0)
+        bm = bm.expand(B, H, -1, -1)
     for b in range(B):
         lk_b = Lk if k_lens is None else max(0, min(int(k_lens[b]), Lk))
         if lk_b == 0:
@@ -89,6 +96,13 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                     raise NotImplementedError("online emulation of causal masking")
                 for j0 in range(0, lk_b, BLKK):
                     j1 = min(j0 + BLKK, lk_b)
+                    if block_mask is not None:
+                        # rows of a 128-row block that does not ask for this tile sit the step out
+                        act = bm[b, h, :, j0 // BLKK].repeat_interleave(128)[:Lq][:, None]
+                        if not bool(act.any()):
+                            continue
+                    else:
+                        act = None
                     sc = (qs_row[b, h][:, None] * k_scale[b, hk, j0 // BLKK]).to(torch.float32)
                     xt = x_f[:, j0:j1]
                     mneg = -(magic * sc)  # fp32
@@ -104,10 +118,14 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                         t = (xt.double() * (8.0 * sc).double() + cp.double()).float()
                         code = torch.round(t).clamp_(0, 126).long()
                         p8 = e4m3fn_decode_table().float()[code]
+                    if act is not None:
+                        m_new = torch.where(act, m_new, m)
+                        alpha = torch.where(act, alpha, torch.ones_like(alpha))
+                        p8 = torch.where(act, p8, torch.zeros_like(p8))
                     l = l * alpha + p8.sum(dim=1, keepdim=True)  # the normaliser sees the rounded P too
                     acc = acc * alpha + p8 @ vf[j0:j1]
                     m = m_new
-                o = acc / l * v_scale[b, hk][None, :]
+                o = torch.where(l > 0, acc / l, torch.zeros_like(acc)) * v_scale[b, hk][None, :]
             else:
                 m = s.amax(dim=1, keepdim=True)
                 p8 = p_to_e4m3(s - m + P_SHIFT, exact_exp2)
@@ -117,7 +135,8 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     return out
 
 
-def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True, exact_exp2=True, k_lens=None):
+def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True, exact_exp2=True, k_lens=None,
+                  block_mask=None):
     """[B, L, H, D] half in, same out: quantise with the oracle quantizer, then emulate."""
     D = q.shape[-1]
     sm_scale = D**-0.5 if sm_scale is None else sm_scale
@@ -125,4 +144,4 @@ def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online
     k_i8, k_scale, _ = quant_k_ref(k, smooth_k=smooth_k)
     v_fp8, v_scale = quant_v_ref(v)
     return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal, online=online,
-                                exact_exp2=exact_exp2, k_lens=k_lens)
+                                exact_exp2=exact_exp2, k_lens=k_lens, block_mask=block_mask)

@@ -29,12 +29,12 @@ def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
     return q.to(dtype), k.to(dtype), v.to(dtype)
 
 
-def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True, k_lens=None):
+def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True, k_lens=None, block_mask=None):
     """The CPU emulation fed with the operands the GPU quantizer actually produced."""
     return sage_emul_from_quant(
         ws.q_i8.cpu()[:, :, :Lq], ws.q_scale.cpu()[:, :, :Lq], untile_k(ws.k_tiles.cpu(), Lk), ws.k_scale.cpu(),
         untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), dtype, exact_exp2=exact_exp2,
-        k_lens=k_lens,
+        k_lens=k_lens, block_mask=block_mask,
     )
 
 
@@ -168,6 +168,62 @@ def test_k_lens_limits_the_keys_per_batch(hip_device, k_lens):
             ws.v_tiles[b, :, t:] = 0x3C
         out_b = sage_ops.attn_fwd(ws, torch.empty_like(qd), k_lens=clamped).cpu()
         assert torch.equal(out_a, out_b)
+
+
+@pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
+@pytest.mark.parametrize("B,Lq,Lk,H,density,seed", [(1, 512, 512, 2, 0.5, 1), (2, 700, 1000, 2, 0.3, 2), (1, 300, 130, 3, 0.6, 3),
+                                                    (1, 1024, 2048, 1, 0.15, 4)])
+def test_block_mask_limits_query_blocks_to_key_tiles(hip_device, B, Lq, Lk, H, density, seed, exact):
+    """mask_id semantics of the reference's block-sparse call (radial_sage_attn.py:150-176): 128 x 64 blocks."""
+    print(f"case B={B} Lq={Lq} Lk={Lk} H={H} density={density} seed={seed} exact={exact}", flush=True)
+    q, k, v = _rand_qkv(B, Lq, Lk, H, H, seed=90 + seed)
+    nq, nk = -(-Lq // 128), -(-Lk // 64)
+    g = torch.Generator().manual_seed(seed)
+    mask = (torch.rand((B, H, nq, nk), generator=g) < density).to(torch.int8)
+    mask[:, :, :, 0] = 1  # every row sees the first tile (the reference's masks keep the first frame too) ...
+    mask[0, 0, nq - 1] = 0  # ... except one query block that sees nothing at all
+    if nq > 1:
+        mask[0, 0, 0] = 0
+        mask[0, 0, 0, nk - 1] = 1  # and one that sees only the last (possibly ragged) tile
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    out = sage_ops.block_sparse_sage2_attn(qd, kd, vd, mask.to(hip_device), workspace=ws, pwl_exp2=not exact).cpu()
+    assert torch.isfinite(out.float()).all()
+    emul = _emul_from_ws(ws, Lq, Lk, q.dtype, exact, block_mask=mask)
+    scale = max(emul.float().abs().max().item(), 1e-3)
+    diff = (out.float() - emul.float()).abs()
+    assert diff.max() <= 2e-2 * scale
+    assert (diff > 1e-2 * scale * 0.5).float().mean() <= 1e-3
+    assert _cos(out, emul) > 0.99999
+    ref = sdpa_ref(q, k, v, block_mask=mask)
+    assert (out[0, 128 * (nq - 1):, 0] == 0).all() and (ref[0, 128 * (nq - 1):, 0] == 0).all()
+    assert _cos(out, ref) >= (COS_MIN if exact else 0.9985)
+    assert (out.float() - ref.float()).abs().max() <= 0.12 * max(ref.float().abs().max().item(), 0.1)
+    # an all-ones mask is the dense kernel's result, bit for bit; a [nq, nk] mask broadcasts
+    dense = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact).cpu()
+    ones = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact, block_mask=torch.ones(nq, nk)).cpu()
+    assert torch.equal(dense, ones)
+    # tiles no row asks for never reach the result: overwrite their quantized images and rerun
+    unused = (mask.view(B, H, -1, nk).sum(dim=2) == 0)  # [B, H, nk]
+    before = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact, block_mask=mask).cpu()
+    ws.k_tiles[unused.to(hip_device)] = 0x55
+    ws.v_tiles[unused.to(hip_device)] = 0x3C
+    after = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact, block_mask=mask).cpu()
+    assert torch.equal(before, after)
+
+
+def test_block_mask_with_k_lens_and_limits(hip_device):
+    B, Lq, Lk, H = 2, 256, 320, 2
+    q, k, v = _rand_qkv(B, Lq, Lk, H, H, seed=55)
+    mask = torch.tensor([[1, 0, 1, 0, 1], [1, 1, 0, 1, 0]], dtype=torch.int8)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, block_mask=mask, k_lens=[150, 320]).cpu()
+    emul = _emul_from_ws(ws, Lq, Lk, q.dtype, block_mask=mask, k_lens=[150, 320])
+    assert _cos(out, emul) > 0.99999
+    assert _cos(out, sdpa_ref(q, k, v, block_mask=mask, k_lens=[150, 320])) >= COS_MIN
+    with pytest.raises(ValueError):
+        sage_ops.sageattn(qd, kd, vd, block_mask=torch.ones(3, 5))  # wrong number of query blocks
 
 
 def test_backend_k_lens_is_opt_in(hip_device):

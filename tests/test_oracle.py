@@ -317,6 +317,52 @@ def test_sdpa_ref_k_lens_equals_cutting_the_batch_entries():
     assert (o_g[1:2].double() - attention_bruteforce_f64(q[1:2], kk[1:2, :7], vv[1:2, :7])).abs().max() < 1e-5
 
 
+def test_sdpa_ref_block_mask_equals_attention_over_the_allowed_keys():
+    """mask_id of the reference's block-sparse call (radial_sage_attn.py:150-176): 128 query rows x 64 keys per
+    entry.  Independent formulation: gather the allowed keys of each query block and run dense attention on them."""
+    B, Lq, Lk, H, D = 2, 300, 200, 2, 16
+    q, k, v = _rand((B, Lq, H, D), 31).float(), _rand((B, Lk, H, D), 32).float(), _rand((B, Lk, H, D), 33).float()
+    g = torch.Generator().manual_seed(34)
+    mask = torch.rand((B, H, 3, 4), generator=g) < 0.5
+    mask[0, 0, 1] = False  # a query block that sees nothing
+    out = sdpa_ref(q, k, v, block_mask=mask)
+    for b in range(B):
+        for h in range(H):
+            for i in range(3):
+                rows = slice(128 * i, min(128 * (i + 1), Lq))
+                cols = torch.cat([torch.arange(64 * j, min(64 * (j + 1), Lk)) for j in range(4) if mask[b, h, i, j]]
+                                 or [torch.zeros(0, dtype=torch.long)])
+                if len(cols) == 0:
+                    assert (out[b, rows, h] == 0).all()
+                    continue
+                want = attention_bruteforce_f64(q[b : b + 1, rows, h : h + 1], k[b : b + 1, cols, h : h + 1], v[b : b + 1, cols, h : h + 1])
+                assert (out[b : b + 1, rows, h : h + 1].double() - want).abs().max() < 1e-5
+    # all-ones mask is dense attention; a [nq, nk] mask broadcasts over batch and heads
+    assert torch.allclose(sdpa_ref(q, k, v, block_mask=torch.ones(3, 4)), sdpa_ref(q, k, v), atol=1e-6)
+    # with k_lens the two restrictions intersect
+    both = sdpa_ref(q, k, v, block_mask=mask, k_lens=[70, 200])
+    cut = sdpa_ref(q[:1], k[:1, :70], v[:1, :70], block_mask=mask[:1, :, :, :2])
+    assert torch.allclose(both[:1], cut, atol=1e-6)
+
+
+def test_sage_emul_block_mask_equals_emulating_the_allowed_tiles():
+    """On the same quantized operands: walking only the allowed key tiles == emulating with the other tiles removed."""
+    B, L, H, D = 1, 256, 1, 128
+    q, k, v = _rand((B, L, H, D), 41), _rand((B, L, H, D), 42), _rand((B, L, H, D), 43)
+    q_i8, q_s = qr.quant_q_ref(q, D**-0.5)
+    k_i8, k_s, _ = qr.quant_k_ref(k)
+    v_f8, v_s = qr.quant_v_ref(v)
+    mask = torch.tensor([[1, 0, 1, 1], [0, 0, 1, 0]])
+    out = sage_emul_from_quant(q_i8, q_s, k_i8, k_s, v_f8, v_s, torch.bfloat16, block_mask=mask)
+    for i in range(2):
+        tiles = [j for j in range(4) if mask[i, j]]
+        cols = torch.cat([torch.arange(64 * j, 64 * (j + 1)) for j in tiles])
+        rows = slice(128 * i, 128 * (i + 1))
+        cut = sage_emul_from_quant(q_i8[:, :, rows], q_s[:, :, rows], k_i8[:, :, cols], k_s[:, :, tiles], v_f8[:, :, cols], v_s,
+                                   torch.bfloat16)
+        assert torch.equal(out[:, rows], cut)
+
+
 def test_sage_emul_k_lens_equals_emulating_the_cut_operands():
     """On the SAME quantized operands, limiting the keys equals dropping the other keys' rows."""
     B, L, H, D = 2, 200, 1, 128
