@@ -76,6 +76,46 @@ WAN_GRIDS = {"cpu_plumbing": (3, 20, 26), "wan5b_720p": (31, 22, 40), "wan14b_48
              "wan14b_720p": (21, 45, 80)}
 
 
+def radial_style_mask(L, grid, blk_q=128, blk_k=64):
+    """A block mask with the structure of the reference's radial masks (attn_mask.py:45-110): every query sees
+    the first frame and its own; the band of allowed in-frame distances halves each time the frame distance
+    doubles.  Built here for timing; it is not the reference's generator."""
+    f, h, wd = grid
+    tpf = h * wd
+    nq, nk = -(-L // blk_q), -(-L // blk_k)
+    qpos = torch.arange(nq) * blk_q + blk_q // 2
+    kpos = torch.arange(nk) * blk_k + blk_k // 2
+    qf, kf = (qpos // tpf).clamp(max=f - 1), (kpos // tpf).clamp(max=f - 1)
+    qi, ki = qpos % tpf, kpos % tpf
+    dist = (qf[:, None] - kf[None, :]).abs()
+    group = torch.where(dist > 0, torch.floor(torch.log2(dist.clamp(min=1).float())) + 1, torch.zeros(()))
+    width = torch.where(dist == 0, torch.full((), float(tpf)), (tpf / 2.0) / torch.pow(2.0, group - 1)).clamp(min=blk_q)
+    mask = (qi[:, None] - ki[None, :]).abs() <= width
+    mask |= (kf == 0)[None, :]
+    return mask.to(torch.int8)
+
+
+def block_sparse_leg(sage_ops, w, ws, out, grid, pwl, iters):
+    """Outside the timed step: the attention kernel driven by a radial-style block mask (128 x 64 blocks)."""
+    mask = radial_style_mask(w.L, grid).to(out.device)
+    density = float(mask.float().mean())
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
+    sage_ops.attn_fwd(ws, out, pwl_exp2=pwl, block_mask=mask)
+    torch.cuda.synchronize()
+    for e in ev:
+        e[0].record()
+        sage_ops.attn_fwd(ws, out, pwl_exp2=pwl, block_mask=mask)
+        e[1].record()
+    torch.cuda.synchronize()
+    ms = sum(e[0].elapsed_time(e[1]) for e in ev) / iters
+    return {
+        "mask": "radial-style, 128x64 blocks, broadcast over heads",
+        "density": round(density, 4),
+        "attn_kernel_ms": round(ms, 4),
+        "tflops_on_kept_blocks": round(w.flops * density / (ms * 1e-3) / 1e12, 2),
+    }
+
+
 def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
     """Outside the timed step: the quantizer with the block's RMSNorm + RoPE applied on the fly
     (q and k taken as the raw projections).  Same 9 N algorithmic bytes as the plain quantizer; what a
@@ -246,6 +286,8 @@ def main() -> int:
         },
     }
     grid = WAN_GRIDS.get(w.name)
+    if grid is not None and w.L <= 131072:
+        rec["block_sparse"] = block_sparse_leg(sage_ops, w, ws, out, grid, args.pwl_exp2, max(3, args.steps // 2))
     if grid is not None and w.B == 1:
         rec["prep_quantizer"] = prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, max(3, args.steps // 2))
     if args.cpu_seconds > 0:
