@@ -28,10 +28,11 @@ def get_backend_mapping() -> dict:
     """Lazy enum -> class registry (built on first use to avoid import cycles, base.py:27-48)."""
     global _ATTN_BACKEND_TO_IMPL
     if _ATTN_BACKEND_TO_IMPL is None:
+        from .radial_sage_attn import RadialSageAttentionImpl
         from .sage_attn import SageAttentionImpl
         from .sdpa import SDPAImpl
 
-        _ATTN_BACKEND_TO_IMPL = {cls.type(): cls for cls in (SageAttentionImpl, SDPAImpl)}
+        _ATTN_BACKEND_TO_IMPL = {cls.type(): cls for cls in (SageAttentionImpl, SDPAImpl, RadialSageAttentionImpl)}
     return _ATTN_BACKEND_TO_IMPL
 
 

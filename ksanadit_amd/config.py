@@ -1,9 +1,9 @@
 """Backend selector for the attention op: enum + frozen config.
 
-Mirrors ksana/config/attention_config.py:23-83 for the two backends this package provides.
+Mirrors ksana/config/attention_config.py:23-104 for the backends this package provides.
 The enum keeps the reference's string values so a config written for the reference selects the
 same backend here; names the reference knows but this package does not build
-(flash / radial / SLA / laser) are accepted by the enum and rejected by ``support()`` exactly
+(flash / SLA / laser) are accepted by the enum and rejected by ``support()`` exactly
 as the reference rejects a backend missing from its platform list
 (attention_config.py:62-68, 79-83).
 """
@@ -25,7 +25,7 @@ class KsanaAttentionBackend(Enum):
     @staticmethod
     def _get_gpu_supported() -> list["KsanaAttentionBackend"]:
         # order is the fallback order of the selector (backends/base.py)
-        return [KsanaAttentionBackend.SAGE_ATTN, KsanaAttentionBackend.TORCH_SDPA]
+        return [KsanaAttentionBackend.SAGE_ATTN, KsanaAttentionBackend.TORCH_SDPA, KsanaAttentionBackend.RADIAL_SAGE_ATTN]
 
     @staticmethod
     def get_supported_list(exclude: list["KsanaAttentionBackend"] | None = None) -> list[str]:
@@ -53,3 +53,23 @@ class KsanaAttentionConfig:
             raise ValueError(
                 f"attention_config {self.backend} not supported in {KsanaAttentionBackend.get_supported_list()}"
             )
+
+
+@dataclass(frozen=True)
+class KsanaRadialSageAttentionConfig(KsanaAttentionConfig):
+    """Settings of the radial block-sparse backend (attention_config.py:86-104)."""
+
+    backend: KsanaAttentionBackend = field(init=False, default=KsanaAttentionBackend.RADIAL_SAGE_ATTN)
+    dense_blocks_num: int = field(default=0)
+    dense_attn_steps: int = field(default=0)
+    decay_factor: float = field(default=0.02)
+    block_size: int = field(default=128)
+    dense_attention_config: KsanaAttentionConfig = field(
+        default=KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN)
+    )
+
+    def __post_init__(self):
+        if self.block_size not in [64, 128]:
+            raise ValueError(f"block_size must be 64 or 128, got {self.block_size}")
+        if not (0 < self.decay_factor < 1):
+            raise ValueError(f"decay_factor must be in range (0, 1), got {self.decay_factor}")

@@ -226,6 +226,37 @@ def test_block_mask_with_k_lens_and_limits(hip_device):
         sage_ops.sageattn(qd, kd, vd, block_mask=torch.ones(3, 5))  # wrong number of query blocks
 
 
+def test_radial_backend_gates_and_masks(hip_device):
+    """radial_sage_attn.py:93-176: dense for early steps / first blocks, else the radial block mask."""
+    from ksanadit_amd.backends.radial_mask import kernel_block_mask, radial_block_mask
+    from ksanadit_amd.backends.radial_sage_attn import RadialSageAttentionImpl
+    from ksanadit_amd.config import KsanaRadialSageAttentionConfig
+
+    B, frames, h, w, H = 1, 6, 16, 16, 2
+    L = frames * h * w  # 1536 tokens, 256 per frame
+    q, k, v = _rand_qkv(B, L, L, H, H, seed=61)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    cfg = KsanaRadialSageAttentionConfig(dense_blocks_num=1, dense_attn_steps=2, decay_factor=0.2, block_size=128)
+    op = pick_attn_op(cfg)(num_heads=H, head_size=128, causal=False)
+    lens = torch.tensor([L], device=hip_device)
+    kw = dict(k_lens=lens, latent_shape=[1, 16, frames, h * 2, w * 2], window_size=(-1, -1), proj_l=None)
+    dense = sage_ops.sageattn(qd, kd, vd).cpu()
+    assert torch.equal(op(qd, kd, vd, step_iter=0, block_id=5, **kw).cpu(), dense)  # early step
+    assert torch.equal(op(qd, kd, vd, step_iter=7, block_id=0, **kw).cpu(), dense)  # first block
+    assert torch.equal(op(qd, kd, vd, step_iter=7, block_id=5, dense_only=True, **kw).cpu(), dense)
+    sparse = op(qd, kd, vd, step_iter=7, block_id=5, **kw).cpu()
+    mask = kernel_block_mask(radial_block_mask(L, L, frames, 128, 0.2), 128, L)
+    assert 0.3 < mask.float().mean() < 1.0 and not torch.equal(sparse, dense)
+    assert _cos(sparse, sdpa_ref(q, k, v, block_mask=mask)) >= COS_MIN
+    impl = op.impl if hasattr(op, "impl") else None
+    assert len(RadialSageAttentionImpl._global_cache) >= 1
+    with pytest.raises(ValueError):  # latent height not a multiple of block_size / 8
+        op(qd, kd, vd, step_iter=7, block_id=5, k_lens=lens, latent_shape=[1, 16, frames, 30, 32])
+    two = torch.tensor([L, L - 1], device=hip_device)
+    with pytest.raises(ValueError):
+        op(qd, kd, vd, step_iter=7, block_id=5, k_lens=two, latent_shape=[1, 16, frames, 32, 32])
+
+
 def test_backend_k_lens_is_opt_in(hip_device):
     """The reference's Sage adaptor drops k_lens (sage_attn.py:58-84): so does the backend unless told otherwise."""
     from ksanadit_amd.backends.sage_attn import SageAttentionImpl

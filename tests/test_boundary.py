@@ -124,12 +124,31 @@ def test_tile_index_maps_are_permutations():
 # ----------------------------------------------------------------------------- selector / op
 def test_enum_values_and_supported_list_follow_the_reference():
     assert KsanaAttentionBackend.SAGE_ATTN.value == "sage_attention" and KsanaAttentionBackend.TORCH_SDPA.value == "torch_sdpa"
-    assert KsanaAttentionBackend.get_supported_list() == ["sage_attention", "torch_sdpa"]
-    assert KsanaAttentionBackend.get_supported_list(exclude=[KsanaAttentionBackend.SAGE_ATTN]) == ["torch_sdpa"]
+    assert KsanaAttentionBackend.get_supported_list() == ["sage_attention", "torch_sdpa", "radial_sage_attention"]
+    assert KsanaAttentionBackend.get_supported_list(exclude=[KsanaAttentionBackend.SAGE_ATTN]) == ["torch_sdpa", "radial_sage_attention"]
     assert KsanaAttentionBackend.support("torch_sdpa") and not KsanaAttentionBackend.support("flash_attention")
     assert KsanaAttentionBackend.support(KsanaAttentionBackend.FLASH_ATTN) and not KsanaAttentionBackend.support(3)
     mapping = get_backend_mapping()
     assert mapping[KsanaAttentionBackend.SAGE_ATTN] is SageAttentionImpl and mapping[KsanaAttentionBackend.TORCH_SDPA] is SDPAImpl
+
+
+def test_radial_config_and_backend_contract_without_gpu():
+    """attention_config.py:86-104 and radial_sage_attn.py:32-59 (constructor checks)."""
+    from ksanadit_amd.backends.radial_sage_attn import RadialSageAttentionImpl
+    from ksanadit_amd.config import KsanaRadialSageAttentionConfig
+
+    cfg = KsanaRadialSageAttentionConfig()
+    assert cfg.backend is KsanaAttentionBackend.RADIAL_SAGE_ATTN and cfg.block_size == 128 and cfg.decay_factor == 0.02
+    assert cfg.dense_attention_config.backend is KsanaAttentionBackend.SAGE_ATTN
+    for bad in ({"block_size": 32}, {"decay_factor": 0.0}, {"decay_factor": 1.0}):
+        with pytest.raises(ValueError):
+            KsanaRadialSageAttentionConfig(**bad)
+    assert get_backend_mapping()[KsanaAttentionBackend.RADIAL_SAGE_ATTN] is RadialSageAttentionImpl
+    assert RadialSageAttentionImpl.type() is KsanaAttentionBackend.RADIAL_SAGE_ATTN
+    if not torch.cuda.is_available():
+        assert RadialSageAttentionImpl.supports(head_size=128) is False
+        with pytest.raises(RuntimeError):
+            RadialSageAttentionImpl(cfg, 2, 128, False, 0.1)
 
 
 def test_config_and_selector_errors():
