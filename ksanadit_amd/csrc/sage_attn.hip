@@ -161,7 +161,15 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   v16f lacc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) lacc[r] = 0.0f;
-  const v8i ones = {0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838};
+  // eight registers on purpose: left as one constant the compiler keeps a single copy and rebuilds
+  // the 8-register operand with seven moves in every step
+  v8i ones;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    int one4 = 0x38383838;
+    pin(one4);
+    ones[r] = one4;
+  }
 
   // kept opaque so the 16 registers stay resident instead of being rebuilt from constants
   // (8 moves) at every tile
@@ -350,9 +358,10 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   //   at step j   O holds tiles <= j-2 relative to max m(j-2); alpha_prev = 2^(m(j-2) - m(j-1))
   //   step j      O *= alpha_prev (rare branch), then O += P(j-1) V(j-1), both relative to m(j-1)
   // LDS ring of 8 stages: tile j-1 (V), j (V next step), j+1 (K), j+2 .. j+4 (arriving).
-  v8i pf_prev = {0, 0, 0, 0, 0, 0, 0, 0};
+  // probabilities of the previous and of the current tile swap registers every step, like s_a / s_b
+  v8i pf_x = {0, 0, 0, 0, 0, 0, 0, 0}, pf_y = {0, 0, 0, 0, 0, 0, 0, 0};
   float alpha_prev = 1.0f;
-  auto tile_step = [&](int j, v16i (&s_cur)[2], v16i (&s_nxt)[2]) {
+  auto tile_step = [&](int j, v16i (&s_cur)[2], v16i (&s_nxt)[2], const v8i& pf_prev, v8i& pf) {
     const uint8_t* kst = smem + ((j + 1) & (kStages - 1)) * kStageBytes;
     const uint8_t* vst = smem + ((j - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
     auto k_frag = [&](int i) { return *reinterpret_cast<const v4i*>(kst + (((i & 1) * 4 + (i >> 1)) * 64 + lane) * 16); };
@@ -384,7 +393,6 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const float c = (kPShift - m_run) + mneg;
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
-    v8i pf;
     int pm[4];
     __builtin_amdgcn_sched_barrier(0);
     // 8 x [S^T MFMA of tile j+1 (32 matrix cycles) | 2 probabilities of tile j]
@@ -435,7 +443,6 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 #pragma unroll
       for (int i = 0; i < 8; ++i) pf[i] &= keep;
     }
-    pf_prev = pf;
     // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
     tile_barrier();
   };
@@ -443,18 +450,19 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   {
     int j = 0;
     for (; j + 2 <= n_main; j += 2) {
-      tile_step(j, s_a, s_b);
-      tile_step(j + 1, s_b, s_a);
+      tile_step(j, s_a, s_b, pf_x, pf_y);
+      tile_step(j + 1, s_b, s_a, pf_y, pf_x);
     }
-    if (j < n_main) tile_step(j, s_a, s_b);
+    if (j < n_main) tile_step(j, s_a, s_b, pf_x, pf_y);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may outlive the workgroup's LDS
   if (n_main > 0) {  // drain: PV of the last pipelined tile
     scale_o(alpha_prev);
     const uint8_t* vst = smem + ((n_main - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
+    const v8i pf_last = (n_main & 1) ? pf_y : pf_x;  // written by the last step
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_prev);
-    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
+    for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_last);
+    lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_last, lacc, 0, 0, 0, 0, 0, 0);
   }
   if (has_tail && mine_at(n_tiles - 1)) {  // ragged last tile, not pipelined: mask keys >= lk
     const int j = nkb - 1, jj = n_tiles - 1;
