@@ -35,6 +35,7 @@ def parse():
     ap.add_argument("--workload", default=None, help="one of ksanadit_amd.workloads.WORKLOADS (default: headline)")
     ap.add_argument("--pwl-exp2", action="store_true", help="piecewise-linear e4m3 code instead of exp2 on the transcendental unit (faster, less accurate)")
     ap.add_argument("--calib-copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (reference point for HBM traffic counters)")
+    ap.add_argument("--skip-extra", action="store_true", help="leave out the block-sparse and norm+RoPE legs (they run after the timed steps)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
     return ap.parse_args()
 
@@ -286,6 +287,8 @@ def main() -> int:
         },
     }
     grid = WAN_GRIDS.get(w.name)
+    if args.skip_extra:
+        grid = None
     if grid is not None and w.L <= 131072:
         rec["block_sparse"] = block_sparse_leg(sage_ops, w, ws, out, grid, args.pwl_exp2, max(3, args.steps // 2))
     if grid is not None and w.B == 1:
