@@ -100,6 +100,8 @@ def block_sparse_leg(sage_ops, w, ws, out, grid, pwl, iters):
     """Outside the timed step: the attention kernel driven by a radial-style block mask (128 x 64 blocks)."""
     mask = radial_style_mask(w.L, grid).to(out.device)
     density = float(mask.float().mean())
+    pairs = mask[: mask.shape[0] // 2 * 2].view(-1, 2, mask.shape[1]).amax(dim=1)  # what a 256-row workgroup walks
+    density_wg = float(pairs.float().mean())
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
     sage_ops.attn_fwd(ws, out, pwl_exp2=pwl, block_mask=mask)
     torch.cuda.synchronize()
@@ -112,6 +114,7 @@ def block_sparse_leg(sage_ops, w, ws, out, grid, pwl, iters):
     return {
         "mask": "radial-style, 128x64 blocks, broadcast over heads",
         "density": round(density, 4),
+        "density_per_256_row_workgroup": round(density_wg, 4),
         "attn_kernel_ms": round(ms, 4),
         "tflops_on_kept_blocks": round(w.flops * density / (ms * 1e-3) / 1e12, 2),
     }
