@@ -62,10 +62,17 @@ def cpu_baseline(workload, target_s: float):
     heads = int(max(1, min(workload.H, target_s * rate / per_head)))
     t = timed(heads)
     flops = per_head * heads
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), model)
+    except OSError:
+        pass
     return {
         "value": round(flops / t / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": cores,
+        "cpu_model": model,
         "kind": "port",
         "sample": f"{workload.name}: {heads} of {workload.H} heads at full L={workload.L}, bf16, one call, {t:.2f} s",
         "ms_per_call_extrapolated": round(t / heads * workload.H * 1e3, 1),
