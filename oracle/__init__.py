@@ -24,6 +24,17 @@ Functions and what pins each of them:
 * ``sage_emul_ref.sage_emul_ref`` dequantised emulation of the fused kernel.  Pinned by its
   distance to ``sdpa_ref`` (it is an approximation by construction) and by the exact
   invariants: V == 1 -> O == 1, key-permutation equivariance, K-offset invariance.
+* ``k_lens`` / ``block_mask`` arguments of ``sdpa_ref`` and ``sage_emul_from_quant``: the per-batch key
+  count of ksana/operations/attention/backends/flash_attn.py:131-139 and the 128 x 64 block mask of
+  backends/radial_sage_attn/radial_sage_attn.py:150-176.  Pinned by an independent formulation each
+  (attention on the cut / gathered operands, float64 brute force), tests/test_oracle.py.
+* ``prep_ref``                    RMSNorm over the token row (ksana/operations/ops.py:62-72) and the 3-axis
+  rotary embedding (ksana/utils/rope.py:61-128, ksana/models/wan/wan_model.py:51-58,677-684).  Pinned by
+  ``torch.nn.functional.rms_norm`` (the routine the reference's default configuration dispatches to),
+  float64 brute force, an independent real-arithmetic form of the rotation and the rotation's
+  invariants (tests/test_prep_oracle.py).  The summation order behind ``mean(x^2)`` is frozen by this
+  repository (not stated by the reference); against the library routine it moves about one bf16 result in
+  10^5 by one ulp.
 
 The arithmetic the reference runs lives in the third-party package ``sageattention``
 (call site ksana/operations/attention/backends/sage_attn.py:75-81), which is neither
