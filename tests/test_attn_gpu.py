@@ -257,6 +257,39 @@ def test_radial_backend_gates_and_masks(hip_device):
         op(qd, kd, vd, step_iter=7, block_id=5, k_lens=two, latent_shape=[1, 16, frames, 32, 32])
 
 
+def test_forward_replays_from_a_hip_graph(hip_device):
+    """The C entry points allocate nothing and only launch kernels, so the whole path can be captured once and
+    replayed: every replay, with eager work and synchronisation in between, must equal the eager result."""
+    q, k, v = _rand_qkv(1, 640, 640, 2, 2, seed=71)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    eager = sage_ops.sageattn(qd, kd, vd, workspace=ws).clone()  # also the warm-up that sets the kernel attributes
+    torch.cuda.synchronize()
+    static_q, static_k, static_v = qd.clone(), kd.clone(), vd.clone()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sage_ops.sageattn(static_q, static_k, static_v, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        static_out = sage_ops.sageattn(static_q, static_k, static_v, workspace=ws)
+    for rep in range(3):
+        ws.blob.fill_(0x5A)  # eager work between replays: the graph must rebuild every intermediate
+        static_out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, eager), f"replay {rep}"
+    # new inputs through the same graph
+    q2, k2, v2 = _rand_qkv(1, 640, 640, 2, 2, seed=72)
+    static_q.copy_(q2.to(hip_device)); static_k.copy_(k2.to(hip_device)); static_v.copy_(v2.to(hip_device))
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(static_out, sage_ops.sageattn(q2.to(hip_device), k2.to(hip_device), v2.to(hip_device)))
+
+
 def test_backend_k_lens_is_opt_in(hip_device):
     """The reference's Sage adaptor drops k_lens (sage_attn.py:58-84): so does the backend unless told otherwise."""
     from ksanadit_amd.backends.sage_attn import SageAttentionImpl
