@@ -30,9 +30,12 @@ def get_backend_mapping() -> dict:
     if _ATTN_BACKEND_TO_IMPL is None:
         from .radial_sage_attn import RadialSageAttentionImpl
         from .sage_attn import SageAttentionImpl
+        from .sage_sla import SageSLAAttentionImpl
         from .sdpa import SDPAImpl
 
-        _ATTN_BACKEND_TO_IMPL = {cls.type(): cls for cls in (SageAttentionImpl, SDPAImpl, RadialSageAttentionImpl)}
+        _ATTN_BACKEND_TO_IMPL = {
+            cls.type(): cls for cls in (SageAttentionImpl, SDPAImpl, RadialSageAttentionImpl, SageSLAAttentionImpl)
+        }
     return _ATTN_BACKEND_TO_IMPL
 
 

@@ -3,7 +3,7 @@
 Mirrors ksana/config/attention_config.py:23-104 for the backends this package provides.
 The enum keeps the reference's string values so a config written for the reference selects the
 same backend here; names the reference knows but this package does not build
-(flash / SLA / laser) are accepted by the enum and rejected by ``support()`` exactly
+(flash / laser) are accepted by the enum and rejected by ``support()`` exactly
 as the reference rejects a backend missing from its platform list
 (attention_config.py:62-68, 79-83).
 """
@@ -25,7 +25,8 @@ class KsanaAttentionBackend(Enum):
     @staticmethod
     def _get_gpu_supported() -> list["KsanaAttentionBackend"]:
         # order is the fallback order of the selector (backends/base.py)
-        return [KsanaAttentionBackend.SAGE_ATTN, KsanaAttentionBackend.TORCH_SDPA, KsanaAttentionBackend.RADIAL_SAGE_ATTN]
+        return [KsanaAttentionBackend.SAGE_ATTN, KsanaAttentionBackend.TORCH_SDPA, KsanaAttentionBackend.RADIAL_SAGE_ATTN,
+                KsanaAttentionBackend.SAGE_SLA]
 
     @staticmethod
     def get_supported_list(exclude: list["KsanaAttentionBackend"] | None = None) -> list[str]:
@@ -73,3 +74,19 @@ class KsanaRadialSageAttentionConfig(KsanaAttentionConfig):
             raise ValueError(f"block_size must be 64 or 128, got {self.block_size}")
         if not (0 < self.decay_factor < 1):
             raise ValueError(f"decay_factor must be in range (0, 1), got {self.decay_factor}")
+
+
+@dataclass(frozen=True)
+class KsanaSageSLAConfig(KsanaAttentionConfig):
+    """Settings of the sparse-linear backend (attention_config.py:107-119): ``topk`` is the share of key blocks
+    every query block keeps."""
+
+    backend: KsanaAttentionBackend = field(init=False, default=KsanaAttentionBackend.SAGE_SLA)
+    dense_attention_config: KsanaAttentionConfig = field(
+        default=KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN)
+    )
+    topk: float = field(default=0.1)
+
+    def __post_init__(self):
+        if not (0 < self.topk < 1):
+            raise ValueError(f"topk must be in range (0, 1), got {self.topk}")

@@ -257,6 +257,34 @@ def test_radial_backend_gates_and_masks(hip_device):
         op(qd, kd, vd, step_iter=7, block_id=5, k_lens=two, latent_shape=[1, 16, frames, 32, 32])
 
 
+def test_sla_backend_sparse_plus_linear(hip_device):
+    """sage_sla.py:141-292: dense when asked, else block-sparse attention on the top-k map plus the projected
+    linear branch."""
+    from ksanadit_amd.backends.sage_sla import linear_branch, topk_block_map
+    from ksanadit_amd.config import KsanaSageSLAConfig
+
+    B, L, H = 1, 1024, 2
+    q, k, v = _rand_qkv(B, L, L, H, H, seed=81)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    op = pick_attn_op(KsanaSageSLAConfig(topk=0.25))(num_heads=H, head_size=128, causal=False)
+    proj = torch.nn.Linear(128, 128, bias=False).to(hip_device).to(torch.bfloat16)
+    torch.nn.init.normal_(proj.weight, std=0.05)
+    assert torch.equal(op(qd, kd, vd, dense_only=True, proj_l=proj).cpu(), sage_ops.sageattn(qd, kd, vd).cpu())
+    with torch.no_grad():
+        out = op(qd, kd, vd, proj_l=proj).cpu()
+    assert out.shape == q.shape and out.dtype == q.dtype
+    # the same composition from the oracle's masked SDPA and torch on the CPU
+    qt, kt, vt = (t.transpose(1, 2) for t in (q, k, v))
+    bmap, kept = topk_block_map(qd.transpose(1, 2), kd.transpose(1, 2), 0.25)
+    assert kept == 4 and (bmap.sum(dim=-1) == 4).all()
+    sparse_ref = sdpa_ref(q, k, v, block_mask=bmap.cpu())
+    with torch.no_grad():
+        lin = proj.cpu().float()(linear_branch(qt.float(), kt.float(), vt.float())).transpose(1, 2)
+    ref = sparse_ref.float() + lin
+    assert _cos(out, ref) >= 0.998
+    assert (out.float() - ref).abs().max() <= 0.15 * max(ref.abs().max().item(), 0.1)
+
+
 def test_forward_replays_from_a_hip_graph(hip_device):
     """The C entry points allocate nothing and only launch kernels, so the whole path can be captured once and
     replayed: every replay, with eager work and synchronisation in between, must equal the eager result."""

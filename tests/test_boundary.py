@@ -124,8 +124,8 @@ def test_tile_index_maps_are_permutations():
 # ----------------------------------------------------------------------------- selector / op
 def test_enum_values_and_supported_list_follow_the_reference():
     assert KsanaAttentionBackend.SAGE_ATTN.value == "sage_attention" and KsanaAttentionBackend.TORCH_SDPA.value == "torch_sdpa"
-    assert KsanaAttentionBackend.get_supported_list() == ["sage_attention", "torch_sdpa", "radial_sage_attention"]
-    assert KsanaAttentionBackend.get_supported_list(exclude=[KsanaAttentionBackend.SAGE_ATTN]) == ["torch_sdpa", "radial_sage_attention"]
+    assert KsanaAttentionBackend.get_supported_list() == ["sage_attention", "torch_sdpa", "radial_sage_attention", "sage_sla"]
+    assert KsanaAttentionBackend.get_supported_list(exclude=[KsanaAttentionBackend.SAGE_ATTN]) == ["torch_sdpa", "radial_sage_attention", "sage_sla"]
     assert KsanaAttentionBackend.support("torch_sdpa") and not KsanaAttentionBackend.support("flash_attention")
     assert KsanaAttentionBackend.support(KsanaAttentionBackend.FLASH_ATTN) and not KsanaAttentionBackend.support(3)
     mapping = get_backend_mapping()
@@ -149,6 +149,40 @@ def test_radial_config_and_backend_contract_without_gpu():
         assert RadialSageAttentionImpl.supports(head_size=128) is False
         with pytest.raises(RuntimeError):
             RadialSageAttentionImpl(cfg, 2, 128, False, 0.1)
+
+
+def test_sla_host_logic_without_gpu():
+    """Block map and linear branch of the sparse-linear backend (sage_sla.py:43-90, 273-282) are plain torch."""
+    from ksanadit_amd.backends.sage_sla import SageSLAAttentionImpl, block_means, linear_branch, topk_block_map
+    from ksanadit_amd.config import KsanaSageSLAConfig
+
+    cfg = KsanaSageSLAConfig(topk=0.25)
+    assert cfg.backend is KsanaAttentionBackend.SAGE_SLA
+    for bad in (0.0, 1.0):
+        with pytest.raises(ValueError):
+            KsanaSageSLAConfig(topk=bad)
+    assert get_backend_mapping()[KsanaAttentionBackend.SAGE_SLA] is SageSLAAttentionImpl
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn((1, 2, 300, 16), generator=g)
+    m = block_means(x, 128)
+    assert m.shape == (1, 2, 3, 16)
+    assert torch.allclose(m[:, :, 0], x[:, :, :128].mean(dim=2), atol=1e-6)
+    assert torch.allclose(m[:, :, 2], x[:, :, 256:].mean(dim=2), atol=1e-6)  # the short last block divides by 44
+    q = torch.randn((1, 2, 512, 16), generator=g)
+    k = torch.randn((1, 2, 1024, 16), generator=g) + 3.0  # the offset must not matter: k is centred first
+    bmap, kept = topk_block_map(q, k, 0.25)
+    assert bmap.shape == (1, 2, 4, 16) and bmap.dtype == torch.int8 and kept == 4
+    assert (bmap.sum(dim=-1) == 4).all()
+    assert torch.equal(bmap, topk_block_map(q, k - 3.0, 0.25)[0])
+    score = block_means(q, 128) @ block_means(k - k.mean(dim=-2, keepdim=True), 64).transpose(-1, -2)
+    chosen_min = torch.where(bmap.bool(), score, torch.full_like(score, float("inf"))).amin(dim=-1)
+    other_max = torch.where(bmap.bool(), torch.full_like(score, float("-inf")), score).amax(dim=-1)
+    assert (chosen_min >= other_max).all()
+    v = torch.randn((1, 2, 1024, 16), generator=g)
+    o = linear_branch(q, k[:, :, :512], v[:, :, :512])
+    # rows of the feature maps sum to one, so V == const gives (almost) that constant back
+    ones = linear_branch(q, k[:, :, :512], torch.full_like(v[:, :, :512], 2.0))
+    assert o.shape == q.shape and ((ones - 2.0).abs() < 1e-3).all()
 
 
 def test_config_and_selector_errors():
