@@ -127,6 +127,21 @@ def block_sparse_leg(sage_ops, w, ws, out, grid, pwl, iters):
     }
 
 
+def causal_leg(sage_ops, w, ws, out, pwl, iters):
+    """Outside the timed step: the same kernel with causal masking (half of the score matrix)."""
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
+    sage_ops.attn_fwd(ws, out, causal=True, pwl_exp2=pwl)
+    torch.cuda.synchronize()
+    for e in ev:
+        e[0].record()
+        sage_ops.attn_fwd(ws, out, causal=True, pwl_exp2=pwl)
+        e[1].record()
+    torch.cuda.synchronize()
+    ms = sum(e[0].elapsed_time(e[1]) for e in ev) / iters
+    kept = (w.L + 1) / (2.0 * w.L)  # fraction of (query, key) pairs on or below the diagonal
+    return {"attn_kernel_ms": round(ms, 4), "tflops_on_kept_pairs": round(w.flops * kept / (ms * 1e-3) / 1e12, 2)}
+
+
 def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
     """Outside the timed step: the quantizer with the block's RMSNorm + RoPE applied on the fly
     (q and k taken as the raw projections).  Same 9 N algorithmic bytes as the plain quantizer; what a
@@ -301,6 +316,7 @@ def main() -> int:
         grid = None
     if grid is not None and w.L <= 131072:
         rec["block_sparse"] = block_sparse_leg(sage_ops, w, ws, out, grid, args.pwl_exp2, max(3, args.steps // 2))
+        rec["causal"] = causal_leg(sage_ops, w, ws, out, args.pwl_exp2, max(3, args.steps // 2))
     if grid is not None and w.B == 1:
         rec["prep_quantizer"] = prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, max(3, args.steps // 2))
     if args.cpu_seconds > 0:

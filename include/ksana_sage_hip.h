@@ -39,7 +39,7 @@ extern "C" {
 /* error codes */
 #define KSANA_SAGE_OK 0
 #define KSANA_SAGE_EINVAL (-1)   /* bad shape, stride, alignment, dtype or null pointer      */
-#define KSANA_SAGE_ENOTSUP (-2)  /* valid request this build does not implement (D != 128, causal) */
+#define KSANA_SAGE_ENOTSUP (-2)  /* valid request this build does not implement (D != 128, causal with Lq != Lk) */
 #define KSANA_SAGE_EHIP (-3)     /* the HIP runtime reported an error at launch               */
 
 /* flags of the attention entry points */
@@ -141,7 +141,10 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], con
 
 /* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
  * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel
- * call (sage_sla.py:237-253, dense form).  causal must be 0 in this build; flags: KSANA_SAGE_FLAG_*.
+ * call (sage_sla.py:237-253, dense form).  flags: KSANA_SAGE_FLAG_*.
+ * causal: non-zero lets query row i attend to keys [0, i] only (the is_causal of sage_attn.py:75-81 and of
+ * sdpa.py:62-79), on top of k_lens and the block mask.  Defined for Lq == Lk (KSANA_SAGE_ENOTSUP otherwise:
+ * for other shapes the libraries anchor the triangle at different corners) and Lk <= 131072.
  * k_lens: NULL, or a device array of B int32: batch b attends to keys [0, k_lens[b]) only
  * (clamped to [0, Lk]; a batch without keys gets zeros).  Same meaning as the k_lens the
  * reference's callers pass (wan_model.py:182-189) and its variable-length backend honours

@@ -56,8 +56,6 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
         if not platform.is_gpu():
             raise RuntimeError("SageAttention backend requested but no HIP device is available.")
         _capi.load()
-        if causal:
-            raise NotImplementedError("SageAttention HIP backend: causal masking is not implemented")
         self.causal = causal
         self.softmax_scale = softmax_scale
         self.dropout = float(extra_impl_args.get("dropout_p", 0.0))

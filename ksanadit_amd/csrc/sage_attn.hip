@@ -108,7 +108,10 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const int xcd = blockIdx.x & 7;
   const int wg = xcd * wg_per_xcd + (blockIdx.x >> 3);
   if (wg >= n_wg) return;
-  const int bh = wg / n_qwg, qwg = wg - bh * n_qwg;
+  const int bh = wg / n_qwg;
+  int qwg = wg - bh * n_qwg;
+  // causal: the later a query block, the more key tiles it walks - start the long ones first
+  if (kSparse && p.causal) qwg = n_qwg - 1 - qwg;
   const int b = bh / p.Hq, h = bh - b * p.Hq;
   const int bhk = b * p.Hkv + h / (p.Hq / p.Hkv);
 
@@ -196,20 +199,27 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   // << 16 | row-1 flag << 17.  The loop below then walks list positions instead of tile
   // numbers; a wave whose row does not ask for a tile zeroes its probabilities for it and
   // leaves its running maximum alone, so the result is exactly the masked softmax.
+  // Causal attention (key <= query row) runs through the same list: the workgroup lists the tiles up
+  // to the one holding its last row, a wave leaves alone the tiles past its own last row, and the one
+  // tile that straddles its rows' diagonal is masked element by element.
   int* s_list = reinterpret_cast<int*>(smem + kStages * kStageBytes + kSparseMaxKeyTiles * 4);
   int n_tiles = nkb;  // loop length: list entries with a mask, key tiles without
+  // a wave's 32 rows start at a multiple of 32, so exactly one 64-key tile holds their diagonal
+  const int my_last = (kSparse && p.causal) ? (q0 >> 6) : 0x7fffffff;
   if constexpr (kSparse) {
     if (wave == 0) {
       const int nqm = (p.Lq + kMaskBlkQ - 1) / kMaskBlkQ;
-      const int8_t* m0 = p.block_mask + b * p.mask_sB + h * p.mask_sH + (int64_t)(2 * qwg) * p.nkb;
+      const bool masked = p.block_mask != nullptr;
+      const int8_t* m0 = masked ? p.block_mask + b * p.mask_sB + h * p.mask_sH + (int64_t)(2 * qwg) * p.nkb : nullptr;
       const bool two = 2 * qwg + 1 < nqm;
+      const int wg_tiles = p.causal ? min(nkb, ((qwg * kAttnQPerWg + kAttnQPerWg - 1) >> 6) + 1) : nkb;
       int base = 0;
-      for (int j0 = 0; j0 < nkb; j0 += 64) {
+      for (int j0 = 0; j0 < wg_tiles; j0 += 64) {
         const int j = j0 + lane;
         int f0 = 0, f1 = 0;
-        if (j < nkb) {
-          f0 = m0[j] != 0;
-          f1 = two && m0[p.nkb + j] != 0;
+        if (j < wg_tiles) {
+          f0 = !masked || m0[j] != 0;
+          f1 = two && (!masked || m0[p.nkb + j] != 0);
         }
         const bool keep = (f0 | f1) != 0;
         const unsigned long long bal = __ballot(keep);
@@ -235,8 +245,43 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     return jj;
   };
   auto mine_at = [&](int jj) -> bool {
-    if constexpr (kSparse) return ((__builtin_amdgcn_readfirstlane(s_list[jj]) >> (16 + (wave >> 2))) & 1) != 0;
+    if constexpr (kSparse) {
+      const int e = __builtin_amdgcn_readfirstlane(s_list[jj]);
+      return ((e >> (16 + (wave >> 2))) & 1) != 0 && (e & 0xffff) <= my_last;
+    }
     return true;
+  };
+  // causal only: list position jj holds the tile on this wave's diagonal
+  auto diag_at = [&](int jj) -> bool {
+    if constexpr (kSparse) return p.causal && tile_of(jj) == my_last;
+    return false;
+  };
+  // scores of keys beyond the row's own position drop below every real score ...
+  auto causal_half = [&](v16i blk, int t) -> v16i {
+    const int row_local = (q0 & 63) + l32;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      // all-ones where the key lies beyond the row
+      const int beyond = (row_local - 4 * hh - (32 * t + 8 * (r >> 2) + (r & 3))) >> 31;
+      blk[r] = (blk[r] & ~beyond) | ((kMagicI - (1 << 22)) & beyond);
+    }
+    return blk;
+  };
+  auto causal_scores = [&](v16i (&blk)[2]) {
+    blk[0] = causal_half(blk[0], 0);
+    blk[1] = causal_half(blk[1], 1);
+  };
+  // ... and their probability bytes are cleared outright (code 0 is +0.0 in e4m3), so that a row
+  // whose scale is zero does not count them either
+  auto causal_probs = [&](v8i& pf) {
+    const int row_local = (q0 & 63) + l32;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      // bytes of the first min(max(n, 0), 4) keys of this dword stay
+      const int n = min(max(row_local - 4 * hh - (32 * (w >> 2) + 8 * (w & 3)) + 1, 0), 4);
+      const unsigned keep = n >= 4 ? 0xffffffffu : ((1u << (8 * n)) - 1u);
+      pf[w] &= (int)keep;
+    }
   };
 
   // ---- asynchronous tile copies: HBM/L2 -> LDS without passing through registers ----------
@@ -346,6 +391,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 
   v16i s_a[2], s_b[2];
   qk_tile(smem, lane, qf, magic, s_a);
+  if (diag_at(0)) causal_scores(s_a);
   int mx_cur = lane_max(s_a);  // this lane's maximum of the tile whose probabilities come next
   float ks_cur = s_ks[0];
 
@@ -423,6 +469,9 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (kSparse) {  // rare, wave-uniform: the next tile is the one on this wave's diagonal
+      if (j + 1 < n_tiles && diag_at(j + 1)) causal_scores(s_nxt);
+    }
     // 4 x [PV MFMA of tile j-1 (64 matrix cycles) | 4 probabilities of tile j | a quarter of
     // the max reduction of tile j+1, whose S^T MFMAs were issued at least one chunk ago]
 #pragma unroll
@@ -442,6 +491,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       const int keep = mine ? -1 : 0;
 #pragma unroll
       for (int i = 0; i < 8; ++i) pf[i] &= keep;
+      if (diag_at(j)) causal_probs(pf);
     }
     // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
     tile_barrier();
@@ -495,6 +545,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         }
         pf[4 * t + g] = w & (int)keep;
       }
+    if (diag_at(jj)) causal_probs(pf);
     const uint8_t* vst = smem + (jj & (kStages - 1)) * kStageBytes + kTileBytes;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf);
@@ -552,7 +603,7 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const int wg_per_xcd = (n_wg + 7) / 8;
   const dim3 grid(wg_per_xcd * 8), block(kThreadsAttn);
   const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
-  if (p.block_mask != nullptr) {
+  if (p.block_mask != nullptr || p.causal) {
     if (p.nkb > kSparseMaxKeyTiles) return hipErrorInvalidValue;
     // tile ring + K scales of the listed tiles + the tile list and its length
     const size_t lds = kStages * kStageBytes + 2 * kSparseMaxKeyTiles * 4 + 1024;

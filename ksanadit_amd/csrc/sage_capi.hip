@@ -84,6 +84,18 @@ int check_mask(const ksana_sage_shape* s, const int8_t* block_mask, const int64_
   return 0;
 }
 
+// Causal masking is defined for self-attention shapes only: with Lq != Lk the libraries disagree on which
+// corner the triangle is anchored to, and no caller of this path needs it.
+int check_causal(const ksana_sage_shape* s, int causal) {
+  if (!causal) return 0;
+  if (s->Lq != s->Lk)
+    return fail(KSANA_SAGE_ENOTSUP, "causal masking needs Lq == Lk (got %d and %d)", s->Lq, s->Lk);
+  if (s->Lk > ksana_sage::kSparseMaxKeyTiles * ksana_sage::kBlkK)
+    return fail(KSANA_SAGE_ENOTSUP, "Lk=%d exceeds %d with causal masking (the tile list is kept in LDS)", s->Lk,
+                ksana_sage::kSparseMaxKeyTiles * ksana_sage::kBlkK);
+  return 0;
+}
+
 int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype, const int64_t q_st[4],
                  const int64_t k_st[4], const int64_t v_st[4], const int64_t o_st[4], const ksana_sage_shape* s,
                  const ksana_sage_prep* prep, const int8_t* block_mask, const int64_t mask_st[2],
@@ -272,7 +284,7 @@ int ksana_sage_attn_fwd_masked(const void* ws, void* o, int dtype, const int64_t
                                int flags, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_mask(s, block_mask, mask_st)) return rc;
-  if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
+  if (int rc = check_causal(s, causal)) return rc;
   if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -294,6 +306,7 @@ int ksana_sage_attn_fwd_masked(const void* ws, void* o, int dtype, const int64_t
   p.block_mask = block_mask;
   p.mask_sB = block_mask ? mask_st[0] : 0;
   p.mask_sH = block_mask ? mask_st[1] : 0;
+  p.causal = causal ? 1 : 0;
   hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
 }
@@ -332,7 +345,7 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
                  const int32_t* k_lens, float sm_scale, int smooth_k, int causal, int flags, void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_mask(s, block_mask, mask_st)) return rc;
-  if (causal) return fail(KSANA_SAGE_ENOTSUP, "causal masking is not implemented");
+  if (int rc = check_causal(s, causal)) return rc;
   // validate everything before the first launch so a bad argument leaves no partial work
   if (int rc = check_tensor("q", q, dtype, q_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_tensor("k", k, dtype, k_st, s->B, s->Lk, s->Hkv)) return rc;

@@ -75,9 +75,10 @@ struct AttnParams {
   // rows attend to the 64 keys; nullptr = dense
   const int8_t* block_mask;
   int64_t mask_sB, mask_sH;  // element strides of the two leading dims (0 broadcasts)
+  int causal;  // 1: query row i attends to keys [0, i] only (on top of k_lens and the block mask)
 };
 constexpr int kMaskBlkQ = 128;           // query rows per mask row (two per workgroup)
-constexpr int kSparseMaxKeyTiles = 2048; // key tiles per head with a block mask (tile list lives in LDS)
+constexpr int kSparseMaxKeyTiles = 2048; // key tiles per head with a block mask or causal masking (tile list lives in LDS)
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s);
 
 }  // namespace ksana_sage

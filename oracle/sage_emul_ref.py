@@ -51,6 +51,8 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     ``k_lens``: batch ``b`` uses keys ``[0, k_lens[b])`` of the quantized operands (online form only).
     ``block_mask`` (``[B|1, H|1, ceil(Lq/128), ceil(Lk/64)]``): query rows ``128 i ..`` walk only the key tiles ``j``
     with a non-zero entry ``(i, j)``; rows without any tile give zeros (online form only).
+    ``causal`` (``Lq == Lk`` only): row ``i`` sees keys ``[0, i]``; in the online form a row sits out the tiles that
+    start after it and sees a prefix of the tile that holds its own position.
     """
     B, H, Lq, D = q_i8.shape
     Hkv, Lk = k_i8.shape[1], k_i8.shape[2]
@@ -76,7 +78,9 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
             s_int = q_i8[b, h].float() @ k_i8[b, hk].float().t()
             s = s_int * (qs_row[b, h][:, None] * ks_col[b, hk][None, :])
             if causal:
-                mask = torch.ones(Lq, Lk, dtype=torch.bool).tril(diagonal=Lk - Lq)
+                if Lq != Lk:
+                    raise NotImplementedError("causal masking with Lq != Lk")
+                mask = torch.ones(Lq, Lk, dtype=torch.bool).tril()
                 s = s.masked_fill(~mask, float("-inf"))
             vf = v_fp8[b, hk].float()
             if online:
@@ -92,21 +96,27 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 m = torch.full((Lq, 1), float("-inf"))
                 l = torch.zeros(Lq, 1)
                 acc = torch.zeros(Lq, D)
-                if causal:
-                    raise NotImplementedError("online emulation of causal masking")
+                rows = torch.arange(Lq)[:, None]
                 for j0 in range(0, lk_b, BLKK):
                     j1 = min(j0 + BLKK, lk_b)
+                    act = None  # rows that take part in this step
                     if block_mask is not None:
                         # rows of a 128-row block that does not ask for this tile sit the step out
                         act = bm[b, h, :, j0 // BLKK].repeat_interleave(128)[:Lq][:, None]
-                        if not bool(act.any()):
-                            continue
-                    else:
-                        act = None
+                    allow = None  # keys of this tile each row may see
+                    if causal:
+                        # key <= row (Lq == Lk); a row before the tile's first key sits the step out, the rows
+                        # on the diagonal see a prefix of the tile
+                        allow = torch.arange(j0, j1)[None, :] <= rows
+                        act = allow[:, :1] if act is None else (act & allow[:, :1])
+                    if act is not None and not bool(act.any()):
+                        continue
                     sc = (qs_row[b, h][:, None] * k_scale[b, hk, j0 // BLKK]).to(torch.float32)
                     xt = x_f[:, j0:j1]
                     mneg = -(magic * sc)  # fp32
-                    m_tile = (xt.amax(dim=1, keepdim=True).double() * sc.double() + mneg.double()).float()  # fma
+                    # a key the row may not see scores magic - 2**22, below every real dot product
+                    xt_max = xt if allow is None else torch.where(allow, xt, torch.tensor(magic - 4194304.0))
+                    m_tile = (xt_max.amax(dim=1, keepdim=True).double() * sc.double() + mneg.double()).float()  # fma
                     m_new = torch.maximum(m, m_tile)
                     alpha = torch.exp2(m - m_new)
                     c = (P_SHIFT - m_new) + mneg
@@ -118,6 +128,8 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                         t = (xt.double() * (8.0 * sc).double() + cp.double()).float()
                         code = torch.round(t).clamp_(0, 126).long()
                         p8 = e4m3fn_decode_table().float()[code]
+                    if allow is not None:
+                        p8 = torch.where(allow, p8, torch.zeros_like(p8))
                     if act is not None:
                         m_new = torch.where(act, m_new, m)
                         alpha = torch.where(act, alpha, torch.ones_like(alpha))

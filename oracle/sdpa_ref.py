@@ -35,14 +35,14 @@ def sdpa_ref(q, k, v, *, scale=None, causal=False, k_lens=None, block_mask=None)
 
 
 def _sdpa_ref_k_lens(q, k, v, scale, causal, k_lens):
-    if causal:
-        raise NotImplementedError("k_lens together with causal masking")
-    B, Lk = k.shape[0], k.shape[1]
+    B, Lq, Lk = k.shape[0], q.shape[1], k.shape[1]
     lens = torch.as_tensor(k_lens, dtype=torch.int64).clamp(0, Lk)
-    keep = torch.arange(Lk)[None, :] < lens[:, None]  # [B, Lk]
+    keep = (torch.arange(Lk)[None, :] < lens[:, None])[:, None, None, :]  # [B, 1, 1, Lk]
+    if causal:  # the triangle anchored at the top-left corner, as is_causal=True defines it
+        keep = keep & torch.ones(Lq, Lk, dtype=torch.bool).tril()
     qt, kt, vt = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
     gqa = qt.shape[1] != kt.shape[1]
-    out = F.scaled_dot_product_attention(qt, kt, vt, attn_mask=keep[:, None, None, :].to(q.device), dropout_p=0.0,
+    out = F.scaled_dot_product_attention(qt, kt, vt, attn_mask=keep.to(q.device), dropout_p=0.0,
                                          scale=scale, **({"enable_gqa": True} if gqa else {}))
     out = out.transpose(1, 2)
     empty = (lens == 0).to(q.device)
@@ -53,8 +53,6 @@ def _sdpa_ref_k_lens(q, k, v, scale, causal, k_lens):
 
 
 def _sdpa_ref_block_mask(q, k, v, scale, causal, k_lens, block_mask, blk_q=128, blk_k=64):
-    if causal:
-        raise NotImplementedError("block_mask together with causal masking")
     B, Lq, H, _ = q.shape
     Lk = k.shape[1]
     m = torch.as_tensor(block_mask) != 0
@@ -62,6 +60,8 @@ def _sdpa_ref_block_mask(q, k, v, scale, causal, k_lens, block_mask, blk_q=128, 
         m = m.unsqueeze(0)
     keep = m.repeat_interleave(blk_q, dim=2)[:, :, :Lq].repeat_interleave(blk_k, dim=3)[:, :, :, :Lk]
     keep = keep.expand(B, H, Lq, Lk)
+    if causal:
+        keep = keep & torch.ones(Lq, Lk, dtype=torch.bool).tril()
     if k_lens is not None:
         lens = torch.as_tensor(k_lens, dtype=torch.int64).clamp(0, Lk)
         keep = keep & (torch.arange(Lk)[None, :] < lens[:, None])[:, None, None, :]

@@ -29,12 +29,12 @@ def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
     return q.to(dtype), k.to(dtype), v.to(dtype)
 
 
-def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True, k_lens=None, block_mask=None):
+def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True, k_lens=None, block_mask=None, causal=False):
     """The CPU emulation fed with the operands the GPU quantizer actually produced."""
     return sage_emul_from_quant(
         ws.q_i8.cpu()[:, :, :Lq], ws.q_scale.cpu()[:, :, :Lq], untile_k(ws.k_tiles.cpu(), Lk), ws.k_scale.cpu(),
         untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), dtype, exact_exp2=exact_exp2,
-        k_lens=k_lens, block_mask=block_mask,
+        k_lens=k_lens, block_mask=block_mask, causal=causal,
     )
 
 
@@ -224,6 +224,65 @@ def test_block_mask_with_k_lens_and_limits(hip_device):
     assert _cos(out, sdpa_ref(q, k, v, block_mask=mask, k_lens=[150, 320])) >= COS_MIN
     with pytest.raises(ValueError):
         sage_ops.sageattn(qd, kd, vd, block_mask=torch.ones(3, 5))  # wrong number of query blocks
+
+
+@pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
+@pytest.mark.parametrize("B,L,H", [(1, 33, 1), (1, 64, 1), (1, 256, 2), (2, 300, 3), (1, 1000, 2), (1, 2048, 1)])
+def test_causal_rows_see_their_own_prefix(hip_device, B, L, H, exact):
+    """is_causal of the reference's call (sage_attn.py:75-81) for self-attention shapes."""
+    print(f"case causal B={B} L={L} H={H} exact={exact}", flush=True)
+    q, k, v = _rand_qkv(B, L, L, H, H, seed=700 + L)
+    q[0, min(5, L - 1)] = 0  # a row whose scores all tie: the keys beyond it must still not count
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, is_causal=True, pwl_exp2=not exact).cpu()
+    assert torch.isfinite(out.float()).all()
+    emul = _emul_from_ws(ws, L, L, q.dtype, exact, causal=True)
+    scale = max(emul.float().abs().max().item(), 1e-3)
+    diff = (out.float() - emul.float()).abs()
+    assert diff.max() <= 2e-2 * scale
+    assert (diff > 1e-2 * scale * 0.5).float().mean() <= 1e-3
+    assert _cos(out, emul) > 0.99999
+    ref = sdpa_ref(q, k, v, causal=True)
+    assert _cos(out, ref) >= (COS_MIN if exact else 0.9985)
+    assert (out.float() - ref.float()).abs().max() <= 0.12 * max(ref.float().abs().max().item(), 0.1)
+    # row 0 sees key 0 only: the output is V[0] after its FP8 round trip
+    assert (out[:, 0].float() - v[:, 0].float()).abs().max() <= 0.07 * v[:, 0].float().abs().max()
+    # keys after a row never reach it: scramble the quantized images of the last key tile and compare the rows before it
+    last = (L - 1) // 64
+    if last > 0:
+        ws.k_tiles[:, :, last] = 0x11
+        ws.v_tiles[:, :, last] = 0x3C
+        again = sage_ops.attn_fwd(ws, torch.empty_like(qd), causal=True, pwl_exp2=not exact).cpu()
+        assert torch.equal(again[:, : 64 * last], out[:, : 64 * last])
+
+
+def test_causal_with_k_lens_block_mask_backend_and_limits(hip_device):
+    B, L, H = 2, 400, 2
+    q, k, v = _rand_qkv(B, L, L, H, H, seed=77)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    lens = [400, 130]
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, is_causal=True, k_lens=lens).cpu()
+    assert _cos(out, _emul_from_ws(ws, L, L, q.dtype, k_lens=lens, causal=True)) > 0.99999
+    assert _cos(out, sdpa_ref(q, k, v, causal=True, k_lens=lens)) >= COS_MIN
+    nq, nk = -(-L // 128), -(-L // 64)
+    mask = (torch.rand((B, H, nq, nk), generator=torch.Generator().manual_seed(78)) < 0.6).to(torch.int8)
+    mask[:, :, :, 0] = 1
+    mask[0, 0, 1] = 0
+    mask[0, 0, 1, 3] = 1  # rows 128..255 of one head see tile 3 (keys 192..255) only: rows 128..191 get zeros
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, is_causal=True, block_mask=mask).cpu()
+    emul = _emul_from_ws(ws, L, L, q.dtype, block_mask=mask, causal=True)
+    assert (out[0, 128:192, 0] == 0).all() and (emul[0, 128:192, 0] == 0).all() and (out[0, 192:256, 0] != 0).any()
+    assert _cos(out, emul) > 0.99999
+    assert _cos(out, sdpa_ref(q, k, v, causal=True, block_mask=mask)) >= COS_MIN
+    # through the operator, next to the SDPA backend with the same constructor arguments
+    sage = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN))(num_heads=H, head_size=128, causal=True)
+    sdpa = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.TORCH_SDPA))(num_heads=H, head_size=128, causal=True)
+    assert _cos(sage(qd, kd, vd).cpu(), sdpa(qd, kd, vd).cpu()) >= COS_MIN
+    # other shapes: the libraries disagree on the corner the triangle hangs from, so the call is refused
+    with pytest.raises(NotImplementedError):
+        sage_ops.sageattn(qd[:, :100], kd, vd, is_causal=True)
 
 
 def test_radial_backend_gates_and_masks(hip_device):

@@ -378,6 +378,59 @@ def test_sage_emul_k_lens_equals_emulating_the_cut_operands():
         assert torch.equal(out[b : b + 1], cut)
 
 
+def test_sdpa_ref_causal_with_k_lens_and_block_mask_row_by_row():
+    """Causal masking on top of the other two restrictions.  Independent formulation: row i alone, attending to
+    the keys it may see, gathered by hand."""
+    B, L, H, D = 2, 150, 2, 16
+    q, k, v = (_rand((B, L, H, D), s).float() for s in (51, 52, 53))
+    lens = [150, 90]
+    mask = torch.tensor([[0, 1, 1], [1, 1, 0]])  # [ceil(150/128), ceil(150/64)]: rows 0..63 see nothing
+    plain = sdpa_ref(q, k, v, causal=True)
+    with_len = sdpa_ref(q, k, v, causal=True, k_lens=lens)
+    with_mask = sdpa_ref(q, k, v, causal=True, block_mask=mask)
+    for b in range(B):
+        for i in (0, 1, 63, 64, 65, 100, 127, 128, 149):
+            row = slice(i, i + 1)
+            want = attention_bruteforce_f64(q[b : b + 1, row], k[b : b + 1, : i + 1], v[b : b + 1, : i + 1])
+            assert (plain[b : b + 1, row].double() - want).abs().max() < 1e-5
+            n = min(i + 1, lens[b])
+            want = attention_bruteforce_f64(q[b : b + 1, row], k[b : b + 1, :n], v[b : b + 1, :n])
+            assert (with_len[b : b + 1, row].double() - want).abs().max() < 1e-5
+            cols = torch.tensor([c for c in range(i + 1) if mask[i // 128, c // 64]], dtype=torch.long)
+            if len(cols) == 0:
+                assert (with_mask[b, i] == 0).all()
+            else:
+                want = attention_bruteforce_f64(q[b : b + 1, row], k[b : b + 1, cols], v[b : b + 1, cols])
+                assert (with_mask[b : b + 1, row].double() - want).abs().max() < 1e-5
+    assert (with_mask[:, :64] == 0).all() and (with_mask[:, 64:] != 0).any()
+
+
+def test_sage_emul_causal_equals_emulating_each_row_on_its_prefix():
+    """On the same quantized operands: row i under causal masking == that row alone with the key count cut to
+    i + 1 (the k_lens form, pinned above by cutting the operands)."""
+    B, L, H, D = 1, 200, 1, 128
+    q, k, v = _rand((B, L, H, D), 61), _rand((B, L, H, D), 62), _rand((B, L, H, D), 63)
+    q_i8, q_s = qr.quant_q_ref(q, D**-0.5)
+    k_i8, k_s, _ = qr.quant_k_ref(k)
+    v_f8, v_s = qr.quant_v_ref(v)
+    for exact in (True, False):
+        out = sage_emul_from_quant(q_i8, q_s, k_i8, k_s, v_f8, v_s, torch.bfloat16, causal=True, exact_exp2=exact)
+        for i in (0, 1, 31, 32, 63, 64, 65, 127, 128, 191, 192, 199):
+            row = slice(i, i + 1)
+            one = sage_emul_from_quant(q_i8[:, :, row], q_s[:, :, row], k_i8, k_s, v_f8, v_s, torch.bfloat16, k_lens=[i + 1],
+                                       exact_exp2=exact)
+            assert torch.equal(out[:, row], one), i
+    # with a block mask the two restrictions intersect: rows 128.. lose tile 2 and with it their own position
+    mask = torch.tensor([[1, 1, 1, 1], [1, 1, 0, 1]])
+    both = sage_emul_from_quant(q_i8, q_s, k_i8, k_s, v_f8, v_s, torch.bfloat16, causal=True, block_mask=mask)
+    ref = sage_emul_from_quant(q_i8, q_s, k_i8, k_s, v_f8, v_s, torch.bfloat16, causal=True)
+    assert torch.equal(both[:, :128], ref[:, :128])
+    cut = sage_emul_from_quant(q_i8[:, :, 128:192], q_s[:, :, 128:192], k_i8[:, :, :128], k_s[:, :, :2], v_f8[:, :, :128], v_s,
+                               torch.bfloat16)
+    assert torch.equal(both[:, 128:192], cut)  # rows 128..191: tiles 0 and 1 whole, tile 2 masked, tile 3 in the future
+    assert _cos(sdpa_ref(q, k, v, causal=True), ref) > 0.999
+
+
 # ------------------------------------------------------------------ emulation of the fused kernel
 def _cos(a, b):
     a, b = a.double().flatten(), b.double().flatten()
