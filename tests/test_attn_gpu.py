@@ -439,3 +439,49 @@ def test_full_size_properties(hip_device, name):
     assert (o1.float() - 1.0).abs().max().item() <= 0.05
     # determinism
     assert torch.equal(out, sage_ops.sageattn(q, k, v))
+
+
+def test_maximum_key_lengths(hip_device):
+    """The longest sequences the library accepts: 262144 keys dense, 131072 with a block mask or causal
+    masking (the per-head tile bookkeeping lives in LDS).  One more key is refused."""
+    g = torch.Generator().manual_seed(4242)
+    # --- dense, Lk = 262144: against the SDPA oracle on the CPU
+    Lq, Lk = 300, 262144
+    print(f"max dense Lq={Lq} Lk={Lk}", flush=True)
+    q = torch.randn((1, Lq, 1, 128), generator=g).mul_(3.0).to(torch.bfloat16)  # peaked rows: a flat softmax over 2^18 keys says little
+    k = torch.randn((1, Lk, 1, 128), generator=g).to(torch.bfloat16)
+    v = torch.randn((1, Lk, 1, 128), generator=g).to(torch.bfloat16)
+    out = sage_ops.sageattn(q.to(hip_device), k.to(hip_device), v.to(hip_device)).cpu()
+    ref = sdpa_ref(q.float(), k.float(), v.float())
+    assert _cos(out, ref) >= COS_MIN
+    with pytest.raises(NotImplementedError):
+        sage_ops.workspace_for(q.to(hip_device), torch.empty((1, Lk + 1, 1, 128), dtype=torch.bfloat16, device=hip_device))
+    # --- block mask, Lk = 131072, the last tile among the kept ones
+    Lq, Lk = 512, 131072
+    print(f"max block mask Lq={Lq} Lk={Lk}", flush=True)
+    k, v = k[:, :Lk], v[:, :Lk]
+    q = torch.randn((1, Lq, 1, 128), generator=g).mul_(3.0).to(torch.bfloat16)
+    mask = (torch.rand((4, 2048), generator=g) < 0.3).to(torch.int8)
+    mask[:, 2047] = 1
+    qd, kd, vd = q.to(hip_device), k.to(hip_device), v.to(hip_device)
+    out = sage_ops.sageattn(qd, kd, vd, block_mask=mask).cpu()
+    assert _cos(out, sdpa_ref(q.float(), k.float(), v.float(), block_mask=mask)) >= COS_MIN
+    with pytest.raises(NotImplementedError):
+        sage_ops.sageattn(qd, torch.cat([kd, kd[:, :1]], dim=1), torch.cat([vd, vd[:, :1]], dim=1),
+                          block_mask=torch.ones(4, 2049, dtype=torch.int8))
+    # --- causal, L = 131072: sampled rows against float64 attention over their prefix
+    L = 131072
+    print(f"max causal L={L}", flush=True)
+    q = torch.randn((1, L, 1, 128), generator=g).mul_(3.0).to(torch.bfloat16)
+    out = sage_ops.sageattn(q.to(hip_device), kd, vd, is_causal=True).cpu()
+    assert torch.isfinite(out.float()).all()
+    rows = [0, 1, 63, 64, 255, 256, 4095, 65535, 65536, 100000, L - 257, L - 256, L - 2, L - 1]
+    got = torch.stack([out[0, i, 0] for i in rows]).double()
+    want = []
+    for i in rows:
+        s = (k[0, : i + 1, 0].double() @ q[0, i, 0].double()) * 128**-0.5
+        want.append(torch.softmax(s, dim=0) @ v[0, : i + 1, 0].double())
+    want = torch.stack(want)
+    assert _cos(got, want) >= COS_MIN
+    for a, b in zip(got, want):  # and row by row, a little looser
+        assert _cos(a, b) >= 0.995
