@@ -285,6 +285,7 @@ def sageattn(
     k_lens=None,
     prep: WanPrep | None = None,
     block_mask=None,
+    out_dtype: torch.dtype | None = None,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
 
@@ -292,6 +293,9 @@ def sageattn(
     ``prep`` (optional, "NHD" only): q and k are the raw projections and the block's RMSNorm + RoPE are applied
     while they are read (see ``WanPrep``).
     ``block_mask`` (optional): block-sparse attention, see ``attn_fwd`` (not together with ``prep``).
+    ``out_dtype`` (optional, fp16 or bf16): write the result in this dtype instead of q's - the cast the Wan block
+    applies before its output projection when the projection's weights want another dtype
+    (ksana/models/wan/wan_model.py:197-204), done in the kernel's epilogue from the fp32 accumulators.
 
     ``pwl_exp2=True`` computes the e4m3 code of every probability directly (exp2 with a
     piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate."""
@@ -316,6 +320,16 @@ def sageattn(
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)
+    if out_dtype is not None and out_dtype != q.dtype:
+        if out_dtype not in _DTYPES:
+            raise ValueError(f"out_dtype must be float16 or bfloat16, got {out_dtype}")
+        # the quantized operands carry no dtype: quantize from q's, write the result in the other
+        quant_q(q, ws, sm_scale, prep=prep)
+        quant_k(k, ws, smooth_k, prep=prep)
+        quant_v(v, ws)
+        out = torch.empty((B, Lq, Hq, D), dtype=out_dtype, device=q.device)
+        attn_fwd(ws, out, causal=is_causal, pwl_exp2=pwl_exp2, k_lens=kl, block_mask=block_mask)
+        return out.transpose(1, 2) if tensor_layout == "HND" else out
     if block_mask is not None:
         if prep is not None:
             raise ValueError("block_mask and prep cannot be combined in one call; quantize with prep, then attn_fwd")

@@ -377,6 +377,34 @@ def test_forward_replays_from_a_hip_graph(hip_device):
     assert torch.equal(static_out, sage_ops.sageattn(q2.to(hip_device), k2.to(hip_device), v2.to(hip_device)))
 
 
+def test_output_dtype_can_differ_from_the_inputs(hip_device):
+    """The cast before the block's output projection (wan_model.py:197-204) folded into the epilogue."""
+    B, L, H = 1, 300, 2
+    q, k, v = _rand_qkv(B, L, L, H, H, seed=808)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    same = sage_ops.sageattn(qd, kd, vd, workspace=ws).cpu()
+    half = sage_ops.sageattn(qd, kd, vd, workspace=ws, out_dtype=torch.float16)
+    assert half.dtype == torch.float16 and half.shape == q.shape and half.is_contiguous()
+    half = half.cpu()
+    # same fp32 accumulators, rounded once to each format: fp16 is the finer one here
+    emul16 = _emul_from_ws(ws, L, L, torch.float16)
+    assert _cos(half, emul16) > 0.99999
+    assert (half.float() - same.float()).abs().max() <= 2.0**-8 * same.float().abs().max()
+    assert torch.equal(sage_ops.sageattn(qd, kd, vd, out_dtype=torch.bfloat16).cpu(), same)
+    with pytest.raises(ValueError):
+        sage_ops.sageattn(qd, kd, vd, out_dtype=torch.float32)
+    from ksanadit_amd.backends.sage_attn import SageAttentionImpl
+    impl = SageAttentionImpl(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN), H, 128, False, 128**-0.5,
+                             out_dtype=torch.float16)
+    assert torch.equal(impl.forward(qd, kd, vd).cpu(), half)
+    # with a block mask and per-batch key counts the same route is taken
+    mask = torch.tensor([[1, 0, 1, 1, 0], [1, 1, 0, 0, 1], [0, 0, 1, 1, 1]], dtype=torch.int8)
+    a = sage_ops.sageattn(qd, kd, vd, block_mask=mask, k_lens=[290], out_dtype=torch.float16).cpu()
+    b = sage_ops.sageattn(qd, kd, vd, block_mask=mask, k_lens=[290]).cpu()
+    assert (a.float() - b.float()).abs().max() <= 2.0**-8 * b.float().abs().max()
+
+
 def test_backend_k_lens_is_opt_in(hip_device):
     """The reference's Sage adaptor drops k_lens (sage_attn.py:58-84): so does the backend unless told otherwise."""
     from ksanadit_amd.backends.sage_attn import SageAttentionImpl
