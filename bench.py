@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--pwl-exp2", action="store_true", help="piecewise-linear e4m3 code instead of exp2 on the transcendental unit (faster, less accurate)")
     ap.add_argument("--calib-copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (reference point for HBM traffic counters)")
     ap.add_argument("--skip-extra", action="store_true", help="leave out the block-sparse and norm+RoPE legs (they run after the timed steps)")
+    ap.add_argument("--skip-block-sparse", action="store_true", help="leave out the block-sparse leg only")
+    ap.add_argument("--skip-causal", action="store_true", help="leave out the causal leg only (it launches the same kernel instantiation as the block-sparse leg)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
     return ap.parse_args()
 
@@ -315,8 +317,10 @@ def main() -> int:
     if args.skip_extra:
         grid = None
     if grid is not None and w.L <= 131072:
-        rec["block_sparse"] = block_sparse_leg(sage_ops, w, ws, out, grid, args.pwl_exp2, max(3, args.steps // 2))
-        rec["causal"] = causal_leg(sage_ops, w, ws, out, args.pwl_exp2, max(3, args.steps // 2))
+        if not args.skip_block_sparse:
+            rec["block_sparse"] = block_sparse_leg(sage_ops, w, ws, out, grid, args.pwl_exp2, max(3, args.steps // 2))
+        if not args.skip_causal:
+            rec["causal"] = causal_leg(sage_ops, w, ws, out, args.pwl_exp2, max(3, args.steps // 2))
     if grid is not None and w.B == 1:
         rec["prep_quantizer"] = prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, max(3, args.steps // 2))
     if args.cpu_seconds > 0:
