@@ -513,3 +513,43 @@ def test_maximum_key_lengths(hip_device):
     assert _cos(got, want) >= COS_MIN
     for a, b in zip(got, want):  # and row by row, a little looser
         assert _cos(a, b) >= 0.995
+
+
+def test_randomized_shapes_and_options(hip_device):
+    """A seeded sweep over shapes and option combinations (GQA, ragged lengths, per-batch key counts, block masks,
+    causal, both exp2 forms, both dtypes), each against the emulation on the same quantized operands."""
+    import random
+
+    rng = random.Random(20240607)
+    for case in range(28):
+        B = rng.choice([1, 1, 2, 3])
+        Hkv = rng.choice([1, 2, 3])
+        Hq = Hkv * rng.choice([1, 1, 2])
+        causal = rng.random() < 0.3
+        Lk = rng.choice([1, 7, 63, 64, 65, 127, 130, 255, 256, 300, 511, 640, 777])
+        Lq = Lk if causal else rng.choice([1, 31, 32, 33, 100, 255, 256, 257, 290, 513])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        exact = rng.random() < 0.6
+        k_lens = [rng.randint(0, Lk + 3) for _ in range(B)] if rng.random() < 0.4 else None
+        mask = None
+        if rng.random() < 0.4:
+            nq, nk = -(-Lq // 128), -(-Lk // 64)
+            g = torch.Generator().manual_seed(case)
+            lead = rng.choice([(), (Hq,), (B, Hq), (B, 1)])
+            mask = (torch.rand((*lead, nq, nk), generator=g) < 0.6).to(torch.int8)
+        print(f"case {case}: B={B} Hq={Hq} Hkv={Hkv} Lq={Lq} Lk={Lk} {dtype} exact={exact} causal={causal} k_lens={k_lens} "
+              f"mask={None if mask is None else tuple(mask.shape)}", flush=True)
+        q, k, v = _rand_qkv(B, Lq, Lk, Hq, Hkv, seed=1000 + case, dtype=dtype)
+        qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+        ws = sage_ops.workspace_for(qd, kd)
+        out = sage_ops.sageattn(qd, kd, vd, workspace=ws, is_causal=causal, pwl_exp2=not exact, k_lens=k_lens,
+                                block_mask=mask).cpu()
+        assert torch.isfinite(out.float()).all()
+        emul = _emul_from_ws(ws, Lq, Lk, dtype, exact, k_lens=k_lens, block_mask=mask, causal=causal)
+        scale = max(emul.float().abs().max().item(), 1e-3)
+        diff = (out.float() - emul.float()).abs()
+        assert diff.max() <= 2e-2 * scale, f"case {case}: max diff {diff.max().item()} vs scale {scale}"
+        assert (diff > 1e-2 * scale * 0.5).float().mean() <= 2e-3, f"case {case}"
+        # rows that see no key are exactly zero in both
+        dead = emul.float().abs().sum(dim=-1) == 0
+        assert (out[dead] == 0).all()
