@@ -18,52 +18,40 @@ from .logger import log
 
 
 class KsanaAttentionOp(nn.Module):
-    def __init__(
-        self,
-        num_heads: int,
-        head_size: int,
-        *,
-        num_kv_heads: int | None = None,
-        softmax_scale: float | None = None,
-        causal: bool = False,
-        attention_config: KsanaAttentionConfig = None,
-    ) -> None:
+    def __init__(self, num_heads: int, head_size: int, *, num_kv_heads: int | None = None,
+                 softmax_scale: float | None = None, causal: bool = False,
+                 attention_config: KsanaAttentionConfig = None) -> None:
         super().__init__()
         if attention_config is None:
             raise ValueError("attention_config should not be None")
-        self.num_heads = num_heads
-        self.head_size = head_size
-        self.num_kv_heads = num_kv_heads or num_heads
-        self.softmax_scale = head_size**-0.5 if softmax_scale is None else softmax_scale
-        self.causal = causal
+        log.debug(f"KsanaAttentionOp with config: {attention_config}")
         self.attention_config = attention_config
+        self.num_heads, self.head_size, self.causal = num_heads, head_size, causal
+        self.num_kv_heads = num_heads if not num_kv_heads else num_kv_heads
+        self.softmax_scale = head_size**-0.5 if softmax_scale is None else softmax_scale
+        # the backend object and the input dtype it was picked for
         self._attn_impl: KsanaAttentionBackendImpl | None = None
         self._attn_impl_dtype: torch.dtype | None = None
-        log.debug(f"KsanaAttentionOp with config: {attention_config}")
 
     @property
     def backend_type(self):
-        return None if self._attn_impl is None else self._attn_impl.type()
+        impl = self._attn_impl
+        return impl.type() if impl is not None else None
 
     def _ensure_impl(self, dtype: torch.dtype) -> None:
-        if self._attn_impl is not None and self._attn_impl_dtype == dtype:
-            return
-        impl_cls = get_attention_backend_impl(
-            attention_config=self.attention_config, head_size=self.head_size, dtype=dtype
-        )
-        self._attn_impl = impl_cls(
-            attention_config=self.attention_config,
-            num_heads=self.num_heads,
-            head_size=self.head_size,
-            causal=self.causal,
-            softmax_scale=self.softmax_scale,
-            num_kv_heads=self.num_kv_heads,
-        )
-        self._attn_impl_dtype = dtype
+        """Pick and build the backend on first use, again when the input dtype changes (a backend may support one
+        dtype and not another)."""
+        if self._attn_impl is None or self._attn_impl_dtype != dtype:
+            cls = get_attention_backend_impl(attention_config=self.attention_config, head_size=self.head_size,
+                                             dtype=dtype)
+            self._attn_impl = cls(attention_config=self.attention_config, num_heads=self.num_heads,
+                                  head_size=self.head_size, causal=self.causal, softmax_scale=self.softmax_scale,
+                                  num_kv_heads=self.num_kv_heads)
+            self._attn_impl_dtype = dtype
 
     @torch.compiler.disable
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, **backend_kwargs) -> torch.Tensor:
-        if not (query.dim() == key.dim() == value.dim() == 4):
+        if any(t.dim() != 4 for t in (query, key, value)):
             raise ValueError("LocalAttentionOp expects tensors shaped [B, L, H, D].")
         self._ensure_impl(query.dtype)
         return self._attn_impl.forward(query, key, value, **backend_kwargs)

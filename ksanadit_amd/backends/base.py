@@ -64,43 +64,35 @@ def get_attention_backend_impl(attention_config: KsanaAttentionConfig, **kwargs)
 
 
 class KsanaAttentionBackendImpl(ABC):
-    """What a backend must provide (base.py:76-128)."""
+    """What a backend provides (base.py:76-128): its enum member, an availability probe that receives ``head_size``
+    and ``dtype``, the constructor below, and ``forward(query, key, value, **kwargs)`` on ``[B, L, H, D]``."""
+
+    attention_config: KsanaAttentionConfig
 
     @abstractmethod
-    def __init__(
-        self,
-        attention_config: KsanaAttentionConfig,
-        num_heads: int,
-        head_size: int,
-        causal: bool,
-        softmax_scale: float,
-        num_kv_heads: int | None = None,
-        **extra_impl_args,
-    ) -> None:
-        raise NotImplementedError
+    def __init__(self, attention_config: KsanaAttentionConfig, num_heads: int, head_size: int, causal: bool,
+                 softmax_scale: float, num_kv_heads: int | None = None, **extra_impl_args) -> None: ...
 
     @staticmethod
     @abstractmethod
-    def type() -> KsanaAttentionBackend:
-        raise NotImplementedError
+    def type() -> KsanaAttentionBackend: ...
 
     @staticmethod
     @abstractmethod
-    def supports(**kwargs) -> bool:
-        raise NotImplementedError
+    def supports(**kwargs) -> bool: ...
 
-    def check_config(self):
-        if KsanaAttentionBackend(self.attention_config.backend) != self.type():
-            raise ValueError(
-                f"Attention config {self.attention_config.backend} does not match implementation type {self.type()}"
-            )
+    @abstractmethod
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, **kwargs) -> torch.Tensor: ...
 
+    def check_config(self) -> None:
+        """A backend built for another backend's config is a programming error (base.py:102-106)."""
+        asked, mine = KsanaAttentionBackend(self.attention_config.backend), self.type()
+        if asked != mine:
+            raise ValueError(f"Attention config {self.attention_config.backend} does not match implementation type {mine}")
+
+    # identity hooks of the reference's interface (base.py:108-118); no caller uses them
     def preprocess_qkv(self, qkv: torch.Tensor) -> torch.Tensor:
         return qkv
 
     def postprocess_output(self, output: torch.Tensor) -> torch.Tensor:
         return output
-
-    @abstractmethod
-    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, **kwargs) -> torch.Tensor:
-        raise NotImplementedError

@@ -15,45 +15,33 @@ from .base import KsanaAttentionBackendImpl
 
 
 class SDPAImpl(KsanaAttentionBackendImpl):
+    """``[B, L, H, D]`` in and out around ``torch.nn.functional.scaled_dot_product_attention``; grouped-query
+    attention is switched on when the head counts differ (sdpa.py:66-75)."""
+
+    def __init__(self, attention_config: KsanaAttentionConfig, num_heads: int, head_size: int, causal: bool,
+                 softmax_scale: float, num_kv_heads: int | None = None, **extra_impl_args) -> None:
+        self.attention_config = attention_config
+        self.check_config()
+        self.causal, self.softmax_scale = causal, softmax_scale
+        self.dropout = float(extra_impl_args.get("dropout_p", 0.0))
+
     @staticmethod
     def type() -> KsanaAttentionBackend:
         return KsanaAttentionBackend.TORCH_SDPA
 
     @staticmethod
     def supports(**_) -> bool:
-        return True
+        return True  # torch runs this anywhere
 
-    def __init__(
-        self,
-        attention_config: KsanaAttentionConfig,
-        num_heads: int,
-        head_size: int,
-        causal: bool,
-        softmax_scale: float,
-        num_kv_heads: int | None = None,
-        **extra_impl_args,
-    ) -> None:
-        self.attention_config = attention_config
-        self.causal = causal
-        self.softmax_scale = softmax_scale
-        self.dropout = float(extra_impl_args.get("dropout_p", 0.0))
-        self.check_config()
-
-    def forward(
-        self,
-        query: torch.Tensor,
-        key: torch.Tensor,
-        value: torch.Tensor,
-        *,
-        q_lens: torch.Tensor = None,
-        k_lens: torch.Tensor = None,
-        dropout_p: float = None,
-        softmax_scale: float = None,
-        **_,
-    ) -> torch.Tensor:
-        p = self.dropout if dropout_p is None else dropout_p
-        s = self.softmax_scale if softmax_scale is None else softmax_scale
-        q, k, v = (t.transpose(1, 2) for t in (query, key, value))
-        extra = {"enable_gqa": True} if q.shape[1] != k.shape[1] else {}
-        out = F.scaled_dot_product_attention(q, k, v, dropout_p=p, is_causal=self.causal, scale=s, **extra)
-        return out.transpose(1, 2)
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, *, q_lens: torch.Tensor = None,
+                k_lens: torch.Tensor = None, dropout_p: float = None, softmax_scale: float = None, **_) -> torch.Tensor:
+        # the per-call values win over the constructor's (sdpa.py:58-60); q_lens / k_lens are accepted and unused
+        options = {
+            "dropout_p": self.dropout if dropout_p is None else dropout_p,
+            "scale": self.softmax_scale if softmax_scale is None else softmax_scale,
+            "is_causal": self.causal,
+        }
+        if query.shape[2] != key.shape[2]:
+            options["enable_gqa"] = True
+        heads_first = [t.transpose(1, 2) for t in (query, key, value)]
+        return F.scaled_dot_product_attention(*heads_first, **options).transpose(1, 2)
