@@ -203,8 +203,10 @@ def test_config_and_selector_errors():
 
 
 def test_no_backend_available_raises_runtime_error(monkeypatch):
-    monkeypatch.setattr(SageAttentionImpl, "supports", staticmethod(lambda **_: False))
-    monkeypatch.setattr(SDPAImpl, "supports", staticmethod(lambda **_: False))
+    from ksanadit_amd.backends.base import get_backend_mapping
+
+    for impl in get_backend_mapping().values():
+        monkeypatch.setattr(impl, "supports", staticmethod(lambda **_: False))
     with pytest.raises(RuntimeError, match="No compatible attention"):
         get_attention_backend_impl(KsanaAttentionConfig(backend="torch_sdpa"), head_size=128, dtype=torch.float16)
 
