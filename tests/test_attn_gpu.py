@@ -398,6 +398,9 @@ def test_output_dtype_can_differ_from_the_inputs(hip_device):
     impl = SageAttentionImpl(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN), H, 128, False, 128**-0.5,
                              out_dtype=torch.float16)
     assert torch.equal(impl.forward(qd, kd, vd).cpu(), half)
+    fast = SageAttentionImpl(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN), H, 128, False, 128**-0.5,
+                             pwl_exp2=True)
+    assert torch.equal(fast.forward(qd, kd, vd).cpu(), sage_ops.sageattn(qd, kd, vd, pwl_exp2=True).cpu())
     # with a block mask and per-batch key counts the same route is taken
     mask = torch.tensor([[1, 0, 1, 1, 0], [1, 1, 0, 0, 1], [0, 0, 1, 1, 1]], dtype=torch.int8)
     a = sage_ops.sageattn(qd, kd, vd, block_mask=mask, k_lens=[290], out_dtype=torch.float16).cpu()
