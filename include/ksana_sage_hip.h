@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 5
+#define KSANA_SAGE_ABI_VERSION 6
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -48,6 +48,8 @@ extern "C" {
                                    /* as rne(8*x + 55.5), i.e. exp2 with a piecewise-linear 3-bit mantissa:   */
                                    /* ~35 % fewer vector-ALU slots (about 1.2x faster), cos-sim to SDPA lower */
                                    /* by ~1.5e-4 and the worst element about 2x further out.                  */
+#define KSANA_SAGE_FLAG_SMOOTH_V 2 /* ksana_sage_forward* only: quantize V with its channel means taken off   */
+                                   /* (see ksana_sage_quant_v_smooth).                                        */
 
 /* rows per int8 scale: Q per token, K per 64 keys (sage_sla.py:190,204 uses (128, 64) off-Hopper;
  * the per-token Q scale is free in this kernel's operand layout and tighter) */
@@ -79,6 +81,8 @@ typedef struct ksana_sage_ws_layout {
   uint64_t v_part;  /* fp32  [B, Hkv, nch, D]: chunk abs-max of V                               */
   uint64_t q_rms;   /* fp32  [B, Lq]: 1/sqrt(mean(q_row^2) + eps), written by the *_prep entry points */
   uint64_t k_rms;   /* fp32  [B, Lk]: the same for the key rows                                 */
+  uint64_t v_mean;  /* fp32  [B, Hkv, D]: channel mean taken off V before scaling (rounded to the input */
+                    /*       dtype; zeros without V smoothing); the attention adds it to its output     */
   int32_t lq_pad;
   int32_t nqb;
   int32_t nkb;
@@ -138,6 +142,15 @@ int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t k_strides[4]
  * Replaces transpose_pad_permute_cuda + scale_fuse_quant_cuda (sage_sla.py:222-228). */
 int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], const ksana_sage_shape* shape,
                        void* workspace, void* stream);
+
+/* The same with V smoothing when smooth_v != 0: the mean of every channel over the Lk rows (summed in the order
+ * of the K mean, rounded to the input dtype) is subtracted in fp32 before the abs-max and the scaling, stored in
+ * the workspace, and added back to the attention output (rows of P sum to one).  A channel that sits far from
+ * zero then spends its e4m3 steps on the deviations instead of on the offset.  The `smooth_v` option of the
+ * library behind the reference's call (sage_attn.py:75-81; off in that call, off by default here); one more
+ * read of V.  smooth_v == 0 is ksana_sage_quant_v. */
+int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[4], const ksana_sage_shape* shape,
+                              int smooth_v, void* workspace, void* stream);
 
 /* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
  * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel

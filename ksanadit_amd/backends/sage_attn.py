@@ -15,6 +15,8 @@ Differences, all deliberate:
   variable-length backend does with the same argument (flash_attn.py:131-139) and what padded batches need;
 * ``out_dtype`` (constructor argument, opt-in): the result is written in that half dtype instead of the query's, which
   folds the cast the Wan block applies before its output projection (wan_model.py:197-204) into the kernel;
+* ``smooth_v`` (constructor argument, opt-in): V is quantized around its channel means, which the kernel adds back to
+  the output - the option of the same name of the library behind the reference's call;
 * ``pwl_exp2`` (constructor argument, opt-in): the kernel's faster form of exp2, about 1.2x the speed at a cosine
   similarity lower by ~1.5e-4;
 * availability: no HIP device -> ``supports()`` is False and the selector moves on, like the
@@ -69,6 +71,8 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
         self.out_dtype = extra_impl_args.get("out_dtype")
         # opt-in: the faster piecewise-linear exp2 of the kernel (slightly less accurate, see sage_ops.sageattn)
         self.pwl_exp2 = bool(extra_impl_args.get("pwl_exp2", False))
+        # opt-in: V quantized around its channel means (see sage_ops.sageattn)
+        self.smooth_v = bool(extra_impl_args.get("smooth_v", False))
         self.attention_config = attention_config
         self.check_config()
 
@@ -78,7 +82,8 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
             query, key, value = (t.to(torch.bfloat16) for t in (query, key, value))
         k_lens = kwargs.get("k_lens") if self.honor_k_lens else None
         output = sageattn(query, key, value, tensor_layout="NHD", is_causal=self.causal, sm_scale=self.softmax_scale,
-                          k_lens=k_lens, out_dtype=self.out_dtype, pwl_exp2=self.pwl_exp2)
+                          k_lens=k_lens, out_dtype=self.out_dtype, pwl_exp2=self.pwl_exp2,
+                          smooth_v=self.smooth_v)
         if self.out_dtype is not None:
             return output
         return output if output.dtype == original_dtype else output.to(original_dtype)

@@ -559,14 +559,21 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   if (q < p.Lq) {
     uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
     const float* vs = p.v_scale + (int64_t)bhk * kD;
+    // the channel means the V quantizer took off come back here (rows of P sum to one); they are zeros
+    // without V smoothing, and a row that saw no key stays zero
+    const float* vm = p.v_mean + (int64_t)bhk * kD;
+    const float keep_mean = inv_l != 0.0f ? 1.0f : 0.0f;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d = 32 * dt + 8 * g + 4 * hh;
         const float4 s4 = *reinterpret_cast<const float4*>(vs + d);
-        store4<DT>(orow + d, oacc[dt][4 * g + 0] * inv_l * s4.x, oacc[dt][4 * g + 1] * inv_l * s4.y,
-                   oacc[dt][4 * g + 2] * inv_l * s4.z, oacc[dt][4 * g + 3] * inv_l * s4.w);
+        const float4 m4 = *reinterpret_cast<const float4*>(vm + d);
+        store4<DT>(orow + d, oacc[dt][4 * g + 0] * inv_l * s4.x + m4.x * keep_mean,
+                   oacc[dt][4 * g + 1] * inv_l * s4.y + m4.y * keep_mean,
+                   oacc[dt][4 * g + 2] * inv_l * s4.z + m4.z * keep_mean,
+                   oacc[dt][4 * g + 3] * inv_l * s4.w + m4.w * keep_mean);
       }
     }
   }

@@ -182,6 +182,7 @@ int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout*
   l.v_part = take(bhk * l.nch * kD * 4);
   l.q_rms = take((uint64_t)s->B * s->Lq * 4);
   l.k_rms = take((uint64_t)s->B * s->Lk * 4);
+  l.v_mean = take(bhk * kD * 4);
   l.total_bytes = off;
   *out = l;
   return 0;
@@ -257,6 +258,11 @@ int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const
 
 int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, void* ws,
                        void* stream) {
+  return ksana_sage_quant_v_smooth(v, dtype, st, s, 0, ws, stream);
+}
+
+int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_v,
+                              void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("v", v, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -264,13 +270,25 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksan
   ksana_sage_workspace_layout(s, &l);
   hipStream_t hs = static_cast<hipStream_t>(stream);
   const ksana_sage::InTensor vt = in_tensor(v, dtype, st);
-  hipError_t e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, 1, ws_at<float>(ws, l.v_part), l.nch, hs);
+  const int bhk = s->B * s->Hkv;
+  float* v_mean = ws_at<float>(ws, l.v_mean);
+  hipError_t e = hipSuccess;
+  if (smooth_v) {
+    e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.v_part), l.nch, hs);
+    if (e != hipSuccess) return hip_fail(e, "v column sum launch");
+  }
+  // the same finalisation as for K: mean rounded to the input dtype, or zeros when smoothing is off
+  e = ksana_sage::launch_k_mean_finalize(ws_at<float>(ws, l.v_part), bhk, smooth_v ? l.nch : 0, s->Lk, dtype,
+                                         smooth_v ? 1 : 0, v_mean, hs);
+  if (e != hipSuccess) return hip_fail(e, "v mean finalize launch");
+  e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, smooth_v ? 2 : 1, ws_at<float>(ws, l.v_part), l.nch, hs,
+                                     nullptr, smooth_v ? v_mean : nullptr);
   if (e != hipSuccess) return hip_fail(e, "v abs-max launch");
   e = ksana_sage::launch_v_scale_finalize(ws_at<float>(ws, l.v_part), s->B * s->Hkv, l.nch,
                                           ws_at<float>(ws, l.v_scale), ws_at<float>(ws, l.v_inv), hs);
   if (e != hipSuccess) return hip_fail(e, "v scale finalize launch");
   e = ksana_sage::launch_quant_v(vt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.v_inv),
-                                 ws_at<uint8_t>(ws, l.v_fp8), hs);
+                                 smooth_v ? v_mean : nullptr, ws_at<uint8_t>(ws, l.v_fp8), hs);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_v launch");
 }
 
@@ -298,6 +316,7 @@ int ksana_sage_attn_fwd_masked(const void* ws, void* o, int dtype, const int64_t
   p.k_scale = ws_at<float>(ws, l.k_scale);
   p.v_tiles = ws_at<uint8_t>(ws, l.v_fp8);
   p.v_scale = ws_at<float>(ws, l.v_scale);
+  p.v_mean = ws_at<float>(ws, l.v_mean);
   p.o = ksana_sage::OutTensor{static_cast<uint16_t*>(o), o_st[0], o_st[1], o_st[2], dtype};
   p.B = s->B, p.Hq = s->Hq, p.Hkv = s->Hkv, p.Lq = s->Lq, p.Lk = s->Lk;
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;
@@ -352,7 +371,8 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
   if (int rc = check_tensor("v", v, dtype, v_st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
-  if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
+  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_SMOOTH_V))
+    return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
   {
     ksana_sage::PrepParams pp;
@@ -365,7 +385,8 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
   }
   if (int rc = ksana_sage_quant_q_prep(q, dtype, q_st, s, prep, sm_scale, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_k_prep(k, dtype, k_st, s, prep, smooth_k, ws, stream)) return rc;
-  if (int rc = ksana_sage_quant_v(v, dtype, v_st, s, ws, stream)) return rc;
-  return ksana_sage_attn_fwd_masked(ws, o, dtype, o_st, s, block_mask, mask_st, k_lens, causal, flags, stream);
+  if (int rc = ksana_sage_quant_v_smooth(v, dtype, v_st, s, flags & KSANA_SAGE_FLAG_SMOOTH_V, ws, stream)) return rc;
+  return ksana_sage_attn_fwd_masked(ws, o, dtype, o_st, s, block_mask, mask_st, k_lens, causal,
+                                    flags & ~KSANA_SAGE_FLAG_SMOOTH_V, stream);
 }
 }  // namespace

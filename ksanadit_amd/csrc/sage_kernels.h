@@ -48,8 +48,9 @@ struct PrepParams {
 hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps, float* inv_rms, hipStream_t s);
 
 // column reductions over the sequence: op 0 = ordered fp32 sum, op 1 = max of |x|
+// op 0: column sums, 1: column max |x|, 2: column max |x - centre[d]| (centre: [B, H, D])
 hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s,
-                              const PrepParams* prep = nullptr);
+                              const PrepParams* prep = nullptr, const float* centre = nullptr);
 hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
                                   hipStream_t s);
 hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s);
@@ -57,8 +58,9 @@ hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, fl
                           float* q_scale, hipStream_t s, const PrepParams* prep = nullptr);
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
                           float* k_scale, hipStream_t s, const PrepParams* prep = nullptr);
-hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, uint8_t* v_tiles,
-                          hipStream_t s);
+// v_mean: nullptr, or the channel means taken off before scaling (V smoothing)
+hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, const float* v_mean,
+                          uint8_t* v_tiles, hipStream_t s);
 
 struct AttnParams {
   const int8_t* q_i8;
@@ -67,6 +69,7 @@ struct AttnParams {
   const float* k_scale;
   const uint8_t* v_tiles;
   const float* v_scale;
+  const float* v_mean;  // [B, Hkv, D] added to every output row that saw a key (zeros without V smoothing)
   OutTensor o;
   int B, Hq, Hkv, Lq, Lk, lq_pad, nkb;
   int exact_exp2;  // 1: exp2 on the transcendental unit; 0: piecewise-linear e4m3 code (faster)

@@ -222,12 +222,15 @@ __global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* _
 // ---------------------------------------------------------------------------------------
 // Column reduction over a chunk of 256 rows.  OP 0: fp32 sum in the frozen order (slot i%32
 // sequential over the chunk's 8 row groups, then an adjacent-pair tree over the 32 slots).
-// OP 1: max |x| (order free).  grid = (nch, H, B).
+// OP 1: max |x| (order free).  OP 2: max |x - centre[d]| over the rows that exist (V smoothing: the
+// centre is the channel mean).  grid = (nch, H, B).
 // ---------------------------------------------------------------------------------------
 template <int DT, int OP, bool PRE>
 __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
                                                                int64_t sH, int H, int L, float* __restrict__ part,
-                                                               int nch, const PrepParams pp) {
+                                                               int nch, const PrepParams pp,
+                                                               const float* __restrict__ centre) {
+  constexpr bool kSum = OP == 0;
   const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const uint16_t* base = x + b * sB + h * sH + c16 * 16;
@@ -240,14 +243,21 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
     if constexpr (PRE) {
       if (row < L) prep16<DT>(rows[i], pp, rl, b, row, h, c16);
     }
+    if constexpr (OP == 2) {
+      if (row < L) {
+        const float* cen = centre + ((int64_t)b * H + h) * kD + c16 * 16;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) rows[i][e] = rows[i][e] - cen[e];
+      }
+    }
   }
   float acc[16];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = OP == 0 ? rows[0][e] : fabsf(rows[0][e]);
+  for (int e = 0; e < 16; ++e) acc[e] = kSum ? rows[0][e] : fabsf(rows[0][e]);
 #pragma unroll
   for (int i = 1; i < kMeanChunk / kSlots; ++i) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = OP == 0 ? acc[e] + rows[i][e] : fmaxf(acc[e], fabsf(rows[i][e]));
+    for (int e = 0; e < 16; ++e) acc[e] = kSum ? acc[e] + rows[i][e] : fmaxf(acc[e], fabsf(rows[i][e]));
   }
   // slots of one wave differ in lane bits 3..5
 #pragma unroll
@@ -255,7 +265,7 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const float o = __shfl_xor(acc[e], m);
-      acc[e] = OP == 0 ? acc[e] + o : fmaxf(acc[e], o);
+      acc[e] = kSum ? acc[e] + o : fmaxf(acc[e], o);
     }
   }
   __shared__ float s_w[4][kD];
@@ -266,9 +276,9 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
   }
   __syncthreads();
   if (t < kD) {
-    const float lo = OP == 0 ? s_w[0][t] + s_w[1][t] : fmaxf(s_w[0][t], s_w[1][t]);
-    const float hi = OP == 0 ? s_w[2][t] + s_w[3][t] : fmaxf(s_w[2][t], s_w[3][t]);
-    part[(((int64_t)b * H + h) * nch + ch) * kD + t] = OP == 0 ? lo + hi : fmaxf(lo, hi);
+    const float lo = kSum ? s_w[0][t] + s_w[1][t] : fmaxf(s_w[0][t], s_w[1][t]);
+    const float hi = kSum ? s_w[2][t] + s_w[3][t] : fmaxf(s_w[2][t], s_w[3][t]);
+    part[(((int64_t)b * H + h) * nch + ch) * kD + t] = kSum ? lo + hi : fmaxf(lo, hi);
   }
 }
 
@@ -502,10 +512,11 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
 // consumes it: chunk (dt = d/32, tt = half of the 64 rows) is 64 lanes x 16 bytes,
 // lane = 32*hh + d%32, byte r <-> row 32*tt + 8*(r/4) + 4*hh + r%4.
 // ---------------------------------------------------------------------------------------
-template <int DT>
+template <int DT, bool CENTRE>
 __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __restrict__ v, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L, int nkb,
                                                            const float* __restrict__ v_inv,
+                                                           const float* __restrict__ v_mean,
                                                            uint8_t* __restrict__ v_tiles) {
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
@@ -516,12 +527,23 @@ __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __res
   float inv[16];
 #pragma unroll
   for (int e = 0; e < 16; ++e) inv[e] = v_inv[bh * kD + c16 * 16 + e];
+  float mean[16];
+  if constexpr (CENTRE) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) mean[e] = v_mean[bh * kD + c16 * 16 + e];
+  }
 #pragma unroll
   for (int i = 0; i < kBlkK / kSlots; ++i) {
     const int r = i * kSlots + slot;
     const int row = blk * kBlkK + r;
     float x[16];
     load_row16<DT>(base + (int64_t)row * sL, row < L, x);
+    if constexpr (CENTRE) {  // rows past the end stay zero
+      if (row < L) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) x[e] = x[e] - mean[e];
+      }
+    }
     uint32_t w[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -596,18 +618,20 @@ hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps,
 }
 
 hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s,
-                              const PrepParams* prep) {
+                              const PrepParams* prep, const float* centre) {
   const dim3 grid(nch, H, B), block(kThreads);
   const PrepParams none{};
   KSANA_DISPATCH_DT(x.dtype, {
-    if (op != 0)
-      col_partial_kernel<DT, 1, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none);
+    if (op == 2)
+      col_partial_kernel<DT, 2, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, centre);
+    else if (op == 1)
+      col_partial_kernel<DT, 1, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
     else if (prep == nullptr)
-      col_partial_kernel<DT, 0, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none);
+      col_partial_kernel<DT, 0, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
-      col_partial_kernel<DT, 0, true><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, pp);
+      col_partial_kernel<DT, 0, true><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, pp, nullptr);
     }
   });
   return hipGetLastError();
@@ -660,11 +684,15 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
   return hipGetLastError();
 }
 
-hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, uint8_t* v_tiles,
-                          hipStream_t s) {
+hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, const float* v_mean,
+                          uint8_t* v_tiles, hipStream_t s) {
   const dim3 grid(nkb, H, B), block(kThreads);
-  KSANA_DISPATCH_DT(v.dtype,
-                    (quant_v_kernel<DT><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, v_inv, v_tiles)));
+  KSANA_DISPATCH_DT(v.dtype, {
+    if (v_mean != nullptr)
+      quant_v_kernel<DT, true><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, v_inv, v_mean, v_tiles);
+    else
+      quant_v_kernel<DT, false><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, v_inv, nullptr, v_tiles);
+  });
   return hipGetLastError();
 }
 

@@ -113,6 +113,12 @@ class SageWorkspace:
 
 
     @property
+    def v_mean(self):
+        """Channel means the V quantizer took off (zeros unless it ran with ``smooth_v``)."""
+        s, l = self.shape, self.layout
+        return self._view(l.v_mean, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
+
+    @property
     def q_rms(self):
         s, l = self.shape, self.layout
         return self._view(l.q_rms, s.B * s.Lq * 4, torch.float32, (s.B, s.Lq))
@@ -210,12 +216,13 @@ def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: Wan
     _capi.check(rc, "ksana_sage_quant_k")
 
 
-def quant_v(v: torch.Tensor, ws: SageWorkspace) -> None:
+def quant_v(v: torch.Tensor, ws: SageWorkspace, smooth_v: bool = False) -> None:
+    """``smooth_v``: take the channel means off before scaling; the attention adds them back to its output."""
     _require_hip(v)
     v = _usable(v)
     lib = _capi.load()
-    rc = lib.ksana_sage_quant_v(v.data_ptr(), _DTYPES[v.dtype], _strides(v), C.byref(ws.shape), ws.ptr,
-                                _stream_ptr(v.device))
+    rc = lib.ksana_sage_quant_v_smooth(v.data_ptr(), _DTYPES[v.dtype], _strides(v), C.byref(ws.shape), int(smooth_v),
+                                       ws.ptr, _stream_ptr(v.device))
     _capi.check(rc, "ksana_sage_quant_v")
 
 
@@ -286,6 +293,7 @@ def sageattn(
     prep: WanPrep | None = None,
     block_mask=None,
     out_dtype: torch.dtype | None = None,
+    smooth_v: bool = False,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
 
@@ -293,6 +301,9 @@ def sageattn(
     ``prep`` (optional, "NHD" only): q and k are the raw projections and the block's RMSNorm + RoPE are applied
     while they are read (see ``WanPrep``).
     ``block_mask`` (optional): block-sparse attention, see ``attn_fwd`` (not together with ``prep``).
+    ``smooth_v``: quantize V with its channel means taken off and add them back to the output - the ``smooth_v``
+    option of the library behind the reference's call (off there, off by default here); worth its extra read of V
+    when V's channels sit far from zero.
     ``out_dtype`` (optional, fp16 or bf16): write the result in this dtype instead of q's - the cast the Wan block
     applies before its output projection when the projection's weights want another dtype
     (ksana/models/wan/wan_model.py:197-204), done in the kernel's epilogue from the fp32 accumulators.
@@ -320,13 +331,14 @@ def sageattn(
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)
+    flags = (_capi.FLAG_PWL_EXP2 if pwl_exp2 else 0) | (_capi.FLAG_SMOOTH_V if smooth_v else 0)
     if out_dtype is not None and out_dtype != q.dtype:
         if out_dtype not in _DTYPES:
             raise ValueError(f"out_dtype must be float16 or bfloat16, got {out_dtype}")
         # the quantized operands carry no dtype: quantize from q's, write the result in the other
         quant_q(q, ws, sm_scale, prep=prep)
         quant_k(k, ws, smooth_k, prep=prep)
-        quant_v(v, ws)
+        quant_v(v, ws, smooth_v)
         out = torch.empty((B, Lq, Hq, D), dtype=out_dtype, device=q.device)
         attn_fwd(ws, out, causal=is_causal, pwl_exp2=pwl_exp2, k_lens=kl, block_mask=block_mask)
         return out.transpose(1, 2) if tensor_layout == "HND" else out
@@ -337,8 +349,8 @@ def sageattn(
         rc = lib.ksana_sage_forward_masked(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
             _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape), mask.data_ptr(), mask_st,
-            None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal),
-            _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
+            None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal), flags, ws.ptr,
+            _stream_ptr(q.device),
         )
         _capi.check(rc, "ksana_sage_forward_masked")
         return out.transpose(1, 2) if tensor_layout == "HND" else out
@@ -346,7 +358,8 @@ def sageattn(
     rc = lib.ksana_sage_forward_prep(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
         _strides(q), _strides(k), _strides(v), _strides(out), C.byref(ws.shape),
-        None if c_prep is None else C.byref(c_prep), None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k), int(is_causal), _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0, ws.ptr, _stream_ptr(q.device),
+        None if c_prep is None else C.byref(c_prep), None if kl is None else kl.data_ptr(), sm_scale, int(smooth_k),
+        int(is_causal), flags, ws.ptr, _stream_ptr(q.device),
     )
     _capi.check(rc, "ksana_sage_forward_prep" if prep is not None else "ksana_sage_forward")
     return out.transpose(1, 2) if tensor_layout == "HND" else out

@@ -142,9 +142,19 @@ def quant_k_ref(k: torch.Tensor, smooth_k: bool = True):
     return xi, scale, km
 
 
-def quant_v_ref(v: torch.Tensor):
-    """v: [B, L, H, D] half -> (v_fp8 [B, H, L, D] float8_e4m3fn, v_scale [B, H, D] fp32)."""
+def quant_v_ref(v: torch.Tensor, smooth_v: bool = False):
+    """v: [B, L, H, D] half -> (v_fp8 [B, H, L, D] float8_e4m3fn, v_scale [B, H, D] fp32), and with ``smooth_v`` a
+    third result, the channel mean [B, H, D] in v's dtype that was taken off before scaling.
+
+    ``smooth_v`` is the V counterpart of the K smoothing: the mean over the sequence (same summation order and rounding
+    as ``k_mean_ref``) is subtracted in fp32, the centred values are quantized, and the attention adds the mean back to
+    its output - rows of P sum to one, so ``P (V - m) + m == P V``.  A channel whose values sit far from zero then
+    spends its eight e4m3 steps per octave on the deviations instead of on the offset."""
     x = _to_bhld_f32(v)
+    vm = None
+    if smooth_v:
+        vm = k_mean_ref(v)
+        x = x - vm.to(torch.float32)[:, :, None, :]
     amax = x.abs().amax(dim=2)  # [B, H, D]
     nz = amax > 0
     safe = torch.where(nz, amax, torch.ones_like(amax))
@@ -152,7 +162,8 @@ def quant_v_ref(v: torch.Tensor):
     scale = torch.where(nz, amax / fmax, torch.zeros_like(amax))
     inv = torch.where(nz, fmax / safe, torch.zeros_like(amax))
     y = (x * inv[:, :, None, :]).clamp_(-FP8_MAX, FP8_MAX)
-    return y.to(torch.float8_e4m3fn), scale
+    codes = y.to(torch.float8_e4m3fn)
+    return (codes, scale, vm) if smooth_v else (codes, scale)
 
 
 def e4m3fn_decode_table() -> torch.Tensor:

@@ -42,7 +42,7 @@ def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
 
 
 def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True,
-                         exact_exp2=True, k_lens=None, block_mask=None):
+                         exact_exp2=True, k_lens=None, block_mask=None, v_mean=None):
     """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
 
     ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
@@ -51,6 +51,8 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     ``k_lens``: batch ``b`` uses keys ``[0, k_lens[b])`` of the quantized operands (online form only).
     ``block_mask`` (``[B|1, H|1, ceil(Lq/128), ceil(Lk/64)]``): query rows ``128 i ..`` walk only the key tiles ``j``
     with a non-zero entry ``(i, j)``; rows without any tile give zeros (online form only).
+    ``v_mean`` (``[B, Hkv, D]``, optional): the channel mean the V quantizer took off (``quant_v_ref(..., smooth_v=True)``);
+    it is added back to every output row that saw at least one key.
     ``causal`` (``Lq == Lk`` only): row ``i`` sees keys ``[0, i]``; in the online form a row sits out the tiles that
     start after it and sees a prefix of the tile that holds its own position.
     """
@@ -137,23 +139,29 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                     l = l * alpha + p8.sum(dim=1, keepdim=True)  # the normaliser sees the rounded P too
                     acc = acc * alpha + p8 @ vf[j0:j1]
                     m = m_new
-                o = torch.where(l > 0, acc / l, torch.zeros_like(acc)) * v_scale[b, hk][None, :]
+                o = acc / l * v_scale[b, hk][None, :]
+                if v_mean is not None:
+                    o = o + v_mean[b, hk].float()[None, :]
+                o = torch.where(l > 0, o, torch.zeros_like(o))
             else:
                 m = s.amax(dim=1, keepdim=True)
                 p8 = p_to_e4m3(s - m + P_SHIFT, exact_exp2)
                 l = p8.sum(dim=1, keepdim=True)
                 o = (p8 @ vf) * v_scale[b, hk][None, :] / l
+                if v_mean is not None:
+                    o = o + v_mean[b, hk].float()[None, :]
             out[b, :, h, :] = o.to(out_dtype)
     return out
 
 
 def sage_emul_ref(q, k, v, *, sm_scale=None, smooth_k=True, causal=False, online=True, exact_exp2=True, k_lens=None,
-                  block_mask=None):
+                  block_mask=None, smooth_v=False):
     """[B, L, H, D] half in, same out: quantise with the oracle quantizer, then emulate."""
     D = q.shape[-1]
     sm_scale = D**-0.5 if sm_scale is None else sm_scale
     q_i8, q_scale = quant_q_ref(q, sm_scale)
     k_i8, k_scale, _ = quant_k_ref(k, smooth_k=smooth_k)
-    v_fp8, v_scale = quant_v_ref(v)
+    v_fp8, v_scale, *rest = quant_v_ref(v, smooth_v=smooth_v)
     return sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, q.dtype, causal=causal, online=online,
-                                exact_exp2=exact_exp2, k_lens=k_lens, block_mask=block_mask)
+                                exact_exp2=exact_exp2, k_lens=k_lens, block_mask=block_mask,
+                                v_mean=rest[0] if rest else None)

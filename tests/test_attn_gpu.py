@@ -408,6 +408,46 @@ def test_output_dtype_can_differ_from_the_inputs(hip_device):
     assert (a.float() - b.float()).abs().max() <= 2.0**-8 * b.float().abs().max()
 
 
+@pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
+def test_v_smoothing_adds_the_mean_back(hip_device, exact):
+    """smooth_v: same attention, V quantized around its channel means.  Against the emulation on the same operands
+    (tight) and against SDPA, where it has to beat the plain path on a V whose channels sit far from zero."""
+    B, Lq, Lk, H = 2, 300, 450, 2
+    q, k, v = _rand_qkv(B, Lq, Lk, H, H, seed=4321)
+    v = (v.float() + torch.linspace(-8, 8, 128)).to(torch.bfloat16)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, smooth_v=True, pwl_exp2=not exact).cpu()
+    emul = sage_emul_from_quant(
+        ws.q_i8.cpu()[:, :, :Lq], ws.q_scale.cpu()[:, :, :Lq], untile_k(ws.k_tiles.cpu(), Lk), ws.k_scale.cpu(),
+        untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), q.dtype, exact_exp2=exact,
+        v_mean=ws.v_mean.cpu())
+    scale = max(emul.float().abs().max().item(), 1e-3)
+    assert (out.float() - emul.float()).abs().max() <= 2e-2 * scale
+    # accuracy: read both paths in fp16 (bf16 resolves 0.06 at |O| = 8, which would hide the difference)
+    ref = sdpa_ref(q.float(), k.float(), v.float())
+    smooth16 = sage_ops.sageattn(qd, kd, vd, smooth_v=True, pwl_exp2=not exact, out_dtype=torch.float16).cpu().float()
+    plain16 = sage_ops.sageattn(qd, kd, vd, pwl_exp2=not exact, out_dtype=torch.float16).cpu().float()
+    err_s, err_p = (smooth16 - ref).abs().mean().item(), (plain16 - ref).abs().mean().item()
+    print(f"mean |o - sdpa|: smooth_v {err_s:.5f}, plain {err_p:.5f}", flush=True)
+    assert err_p > 2 * err_s
+    off = torch.linspace(-8, 8, 128)
+    assert _cos(smooth16 - off, ref - off) >= 0.99 > _cos(plain16 - off, ref - off)
+    # rows that see no key stay zero (no mean added), with per-batch key counts and a block mask
+    mask = torch.ones((3, 8), dtype=torch.int8)
+    mask[1] = 0
+    o2 = sage_ops.sageattn(qd, kd, vd, smooth_v=True, block_mask=mask, k_lens=[450, 0], pwl_exp2=not exact).cpu()
+    assert (o2[:, 128:256] == 0).all() and (o2[1] == 0).all() and (o2[0, :128] != 0).any()
+    assert torch.equal(o2[0, :128], out[0, :128]) and torch.equal(o2[0, 256:], out[0, 256:])
+    # through the backend and with another output dtype
+    from ksanadit_amd.backends.sage_attn import SageAttentionImpl
+    impl = SageAttentionImpl(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN), H, 128, False, 128**-0.5,
+                             smooth_v=True, pwl_exp2=not exact)
+    assert torch.equal(impl.forward(qd, kd, vd).cpu(), out)
+    half = sage_ops.sageattn(qd, kd, vd, smooth_v=True, pwl_exp2=not exact, out_dtype=torch.float16).cpu()
+    assert (half.float() - out.float()).abs().max() <= 2.0**-7 * out.float().abs().max()
+
+
 def test_backend_k_lens_is_opt_in(hip_device):
     """The reference's Sage adaptor drops k_lens (sage_attn.py:58-84): so does the backend unless told otherwise."""
     from ksanadit_amd.backends.sage_attn import SageAttentionImpl

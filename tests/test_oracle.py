@@ -297,6 +297,46 @@ def test_quant_v_properties():
     assert (z8.float() == 0).all() and (zs == 0).all()
 
 
+def test_quant_v_smoothing_centres_before_scaling_and_attention_adds_the_mean_back():
+    """smooth_v: the channel mean is the K-mean function (pinned above) applied to V; the codes are those of the
+    plain quantizer fed with the centred values; a constant added to a channel moves the attention output by that
+    constant and nothing else, where without smoothing it costs the channel its resolution."""
+    v = (_rand((2, 200, 2, 128), 71, std=1.0).float() + torch.linspace(-6, 6, 128)).to(torch.bfloat16)
+    v8, vs, vm = qr.quant_v_ref(v, smooth_v=True)
+    assert vm.dtype == v.dtype and torch.equal(vm, qr.k_mean_ref(v))
+    centred = v.float() - vm.float()[:, None]  # [B, L, H, D], exact in fp32 here
+    amax = centred.abs().amax(dim=1)
+    assert torch.equal(vs, amax / torch.full_like(amax, 448.0))
+    inv = torch.full_like(amax, 448.0) / amax
+    want = (centred * inv[:, None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).permute(0, 2, 1, 3)
+    assert torch.equal(v8.view(torch.uint8), want.contiguous().view(torch.uint8))
+    assert (v8.float().abs().amax(dim=2) == 448.0).all()
+    # dequantised + mean reproduces V to e4m3 precision of the DEVIATION, not of the value
+    deq = v8.float() * vs[:, :, None, :] + vm.float()[:, :, None, :]
+    x = v.permute(0, 2, 1, 3).float()
+    dev = (x - vm.float()[:, :, None, :]).abs()
+    assert ((deq - x).abs() <= dev * 2**-4 + vs[:, :, None, :] * 2**-9 + 1e-6).all()
+    # plain call unchanged: two results, no centring
+    plain8, plain_s = qr.quant_v_ref(v)
+    assert torch.equal(plain_s, v.float().abs().amax(dim=1) / 448.0)
+    # attention: offsetting V by a per-channel constant offsets O by it
+    q, k = _rand((2, 200, 2, 128), 72), _rand((2, 200, 2, 128), 73)
+    base = _rand((2, 200, 2, 128), 74)
+    off = torch.linspace(-8, 8, 128)
+    shifted = (base.float() + off).to(torch.bfloat16)
+    ref = sdpa_ref(q.float(), k.float(), shifted.float())
+    smooth = sage_emul_ref(q, k, shifted, smooth_v=True).float()
+    plain = sage_emul_ref(q, k, shifted).float()
+    err_s, err_p = (smooth - ref).abs().max().item(), (plain - ref).abs().max().item()
+    assert err_s < 0.06 and err_p > 2 * err_s, (err_s, err_p)
+    cs, cp = _cos(smooth - off, ref - off), _cos(plain - off, ref - off)
+    assert cs > 0.99 and (1 - cp) > 4 * (1 - cs), (cs, cp)
+    # V == const: the centred values are zero, the scale is zero, the output is the constant
+    c = torch.full((1, 70, 1, 128), 3.0, dtype=torch.bfloat16)
+    o = sage_emul_ref(_rand((1, 70, 1, 128), 75), _rand((1, 70, 1, 128), 76), c, smooth_v=True)
+    assert (o.float() == 3.0).all()
+
+
 def test_sdpa_ref_k_lens_equals_cutting_the_batch_entries():
     """flash_attn.py:131-139 builds batch b from key[b, :k_lens[b]]: the masked oracle must equal attention on the
     cut tensors, entry by entry (an independent formulation: slicing instead of masking)."""

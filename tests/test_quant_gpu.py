@@ -110,3 +110,34 @@ def test_quantizer_bit_exact_workloads(hip_device, name, heads, seq):
     print(f"workload {name} heads={heads}", flush=True)
     q, k, v = make_inputs(name, heads=heads, seq=seq)
     _check_against_oracle(q, k, v, hip_device)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,H", [(1, 64, 1), (2, 130, 2), (1, 1000, 3), (1, 257, 1)])
+def test_v_smoothing_bit_exact(hip_device, B, L, H, dtype):
+    """smooth_v: channel mean (order and rounding of the K mean), abs-max and codes of the centred values, zero
+    padding, and a workspace without smoothing reads zeros where the mean would be."""
+    print(f"case smooth_v B={B} L={L} H={H} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(31 * L + H)
+    v = (1.3 * torch.randn((B, L, H, 128), generator=g) + 5.0 * torch.randn((1, 1, H, 128), generator=g)).to(dtype)
+    v[:, :, :, 7] = 2.5  # a constant channel: centred values, scale and codes are all zero
+    vd = v.to(hip_device)
+    ws = sage_ops.workspace_for(vd, vd)
+    ws.blob.fill_(0xA5)
+    sage_ops.quant_v(vd, ws, smooth_v=True)
+    torch.cuda.synchronize()
+    v8, vs, vm = qr.quant_v_ref(v, smooth_v=True)
+    assert torch.equal(ws.v_mean.cpu(), vm.float()), "v_mean differs"
+    assert torch.equal(ws.v_scale.cpu(), vs), "v_scale differs"
+    tiles = ws.v_tiles.cpu()
+    assert torch.equal(untile_v(tiles, L), v8.view(torch.uint8)), "v_fp8 differs"
+    nkb = tiles.shape[2]
+    if nkb * 64 > L:
+        assert torch.count_nonzero(untile_v(tiles, nkb * 64)[:, :, L:]) == 0, "v padding rows not zero"
+    assert (ws.v_scale.cpu()[:, :, 7] == 0).all() and (ws.v_mean.cpu()[:, :, 7] == 2.5).all()
+    # without smoothing: the plain codes, and zeros in the mean slot
+    sage_ops.quant_v(vd, ws)
+    torch.cuda.synchronize()
+    p8, ps = qr.quant_v_ref(v)
+    assert torch.count_nonzero(ws.v_mean.cpu()) == 0
+    assert torch.equal(ws.v_scale.cpu(), ps) and torch.equal(untile_v(ws.v_tiles.cpu(), L), p8.view(torch.uint8))
