@@ -21,6 +21,10 @@ Functions and what pins each of them:
 * ``quant_ref.quant_v_ref``       per-channel FP8 e4m3fn V (sage_sla.py:222-228).  Pinned by
   an exhaustive 256-entry decode table built from the format definition, round-trip
   exactness, saturation at +-448 and the scalar second implementation.
+  With ``smooth_v`` the channel mean (the K-mean function, pinned above) is taken off first and returned;
+  pinned by recomputing the codes from the centred values with the plain rule, by the dequantisation bound on
+  the deviation, and by the attention identity ``P (V - m) + m == P V`` (a per-channel offset of V moves the
+  emulated output by that offset, tests/test_oracle.py).
 * ``sage_emul_ref.sage_emul_ref`` dequantised emulation of the fused kernel.  Pinned by its
   distance to ``sdpa_ref`` (it is an approximation by construction) and by the exact
   invariants: V == 1 -> O == 1, key-permutation equivariance, K-offset invariance.
