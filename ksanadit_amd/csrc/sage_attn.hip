@@ -440,6 +440,9 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     int pm[4];
+    // The S^T chunks are short (a 32-cycle MFMA each): a wave inside them goes ahead of the SIMD's other
+    // wave, which is usually in its PV chunks and has 64-cycle MFMAs to hide behind (measured: -1.3 %).
+    __builtin_amdgcn_s_setprio(1);
     __builtin_amdgcn_sched_barrier(0);
     // 8 x [S^T MFMA of tile j+1 (32 matrix cycles) | 2 probabilities of tile j]
 #pragma unroll
@@ -472,6 +475,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     if constexpr (kSparse) {  // rare, wave-uniform: the next tile is the one on this wave's diagonal
       if (j + 1 < n_tiles && diag_at(j + 1)) causal_scores(s_nxt);
     }
+    __builtin_amdgcn_s_setprio(0);
     // 4 x [PV MFMA of tile j-1 (64 matrix cycles) | 4 probabilities of tile j | a quarter of
     // the max reduction of tile j+1, whose S^T MFMAs were issued at least one chunk ago]
 #pragma unroll
