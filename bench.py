@@ -304,7 +304,7 @@ def main() -> int:
             "traffic": ATTN_TRAFFIC_BYTES.get(w.name),
         },
         "quantizer_roofline": {
-            "kernels": "col_partial x2, finalize x3, quant_q, quant_k, quant_v",
+            "kernels": "col_partial x2, finalize x2, quant_q, quant_k, quant_v",
             "bound": "hbm",
             "achieved": round(quant_gbs, 1),
             "peak": HBM_PEAK_GBS,

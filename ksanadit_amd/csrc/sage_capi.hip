@@ -276,16 +276,17 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], con
   if (smooth_v) {
     e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.v_part), l.nch, hs);
     if (e != hipSuccess) return hip_fail(e, "v column sum launch");
+    // the same finalisation as for K: the mean rounded to the input dtype
+    e = ksana_sage::launch_k_mean_finalize(ws_at<float>(ws, l.v_part), bhk, l.nch, s->Lk, dtype, 1, v_mean, hs);
+    if (e != hipSuccess) return hip_fail(e, "v mean finalize launch");
   }
-  // the same finalisation as for K: mean rounded to the input dtype, or zeros when smoothing is off
-  e = ksana_sage::launch_k_mean_finalize(ws_at<float>(ws, l.v_part), bhk, smooth_v ? l.nch : 0, s->Lk, dtype,
-                                         smooth_v ? 1 : 0, v_mean, hs);
-  if (e != hipSuccess) return hip_fail(e, "v mean finalize launch");
   e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, smooth_v ? 2 : 1, ws_at<float>(ws, l.v_part), l.nch, hs,
                                      nullptr, smooth_v ? v_mean : nullptr);
   if (e != hipSuccess) return hip_fail(e, "v abs-max launch");
+  // without smoothing the mean slot is cleared here: the attention adds whatever it holds
   e = ksana_sage::launch_v_scale_finalize(ws_at<float>(ws, l.v_part), s->B * s->Hkv, l.nch,
-                                          ws_at<float>(ws, l.v_scale), ws_at<float>(ws, l.v_inv), hs);
+                                          ws_at<float>(ws, l.v_scale), ws_at<float>(ws, l.v_inv),
+                                          smooth_v ? nullptr : v_mean, hs);
   if (e != hipSuccess) return hip_fail(e, "v scale finalize launch");
   e = ksana_sage::launch_quant_v(vt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.v_inv),
                                  smooth_v ? v_mean : nullptr, ws_at<uint8_t>(ws, l.v_fp8), hs);

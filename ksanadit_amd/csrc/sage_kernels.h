@@ -53,7 +53,9 @@ hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, fl
                               const PrepParams* prep = nullptr, const float* centre = nullptr);
 hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
                                   hipStream_t s);
-hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s);
+// zero_mean: nullptr, or the [BH, D] mean slot to clear (V quantized without smoothing)
+hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, float* zero_mean,
+                                   hipStream_t s);
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
                           float* q_scale, hipStream_t s, const PrepParams* prep = nullptr);
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,

@@ -323,9 +323,11 @@ __global__ __launch_bounds__(kFinThreads) void k_mean_finalize_kernel(const floa
   }
 }
 
+// chunk abs-max -> scale and its inverse; `zero_mean` (optional) is the mean slot to clear when V is not smoothed
 __global__ __launch_bounds__(kFinThreads) void v_scale_finalize_kernel(const float* __restrict__ part, int nch,
                                                                        float* __restrict__ v_scale,
-                                                                       float* __restrict__ v_inv) {
+                                                                       float* __restrict__ v_inv,
+                                                                       float* __restrict__ zero_mean) {
   __shared__ float s_part[kFinMaxChunks * kD];
   const int bh = blockIdx.x;
   const float amax = combine_partials<1>(part + (int64_t)bh * nch * kD, nch, s_part);
@@ -333,6 +335,7 @@ __global__ __launch_bounds__(kFinThreads) void v_scale_finalize_kernel(const flo
     const bool nz = amax > 0.0f;
     v_scale[bh * kD + threadIdx.x] = nz ? __fdiv_rn(amax, 448.0f) : 0.0f;
     v_inv[bh * kD + threadIdx.x] = nz ? __fdiv_rn(448.0f, amax) : 0.0f;
+    if (zero_mean != nullptr) zero_mean[bh * kD + threadIdx.x] = 0.0f;
   }
 }
 
@@ -643,8 +646,9 @@ hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int
   return hipGetLastError();
 }
 
-hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, hipStream_t s) {
-  v_scale_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, v_scale, v_inv);
+hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, float* zero_mean,
+                                   hipStream_t s) {
+  v_scale_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, v_scale, v_inv, zero_mean);
   return hipGetLastError();
 }
 
