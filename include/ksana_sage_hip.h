@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 6
+#define KSANA_SAGE_ABI_VERSION 7
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -83,6 +83,9 @@ typedef struct ksana_sage_ws_layout {
   uint64_t k_rms;   /* fp32  [B, Lk]: the same for the key rows                                 */
   uint64_t v_mean;  /* fp32  [B, Hkv, D]: channel mean taken off V before scaling (rounded to the input */
                     /*       dtype; zeros without V smoothing); the attention adds it to its output     */
+  uint64_t split_o; /* fp32  [256, 256, D]: scratch of the attention kernel - unnormalised accumulators */
+                    /*       of workgroups whose key loop was cut into runs (see ksana_sage_attn_fwd)   */
+  uint64_t split_ml;/* fp32  [256, 256, 2]: their running maxima and row sums                           */
   int32_t lq_pad;
   int32_t nqb;
   int32_t nkb;
@@ -155,6 +158,11 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[
 /* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
  * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel
  * call (sage_sla.py:237-253, dense form).  flags: KSANA_SAGE_FLAG_*.
+ * When the number of 256-row query blocks times heads leaves a small remainder against the number of compute units,
+ * the workgroups of that remainder are cut into runs of key tiles that fill the chip together, and a second small
+ * kernel merges the runs (dense, non-causal calls only); the result is the same attention within rounding, and
+ * repeated calls give identical bits.  The quantized operands in the workspace are only read; the runs' scratch
+ * (split_o, split_ml) is the one part of it this call writes.
  * causal: non-zero lets query row i attend to keys [0, i] only (the is_causal of sage_attn.py:75-81 and of
  * sdpa.py:62-79), on top of k_lens and the block mask.  Defined for Lq == Lk (KSANA_SAGE_ENOTSUP otherwise:
  * for other shapes the libraries anchor the triangle at different corners) and Lk <= 131072.
@@ -163,7 +171,7 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[
  * reference's callers pass (wan_model.py:182-189) and its variable-length backend honours
  * (flash_attn.py:131-139); the reference's Sage adaptor drops the argument (sage_attn.py:58-84),
  * which is what NULL reproduces.  The quantizers always see all Lk rows. */
-int ksana_sage_attn_fwd(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
+int ksana_sage_attn_fwd(void* workspace, void* o, int dtype, const int64_t o_strides[4],
                         const ksana_sage_shape* shape, const int32_t* k_lens, int causal, int flags, void* stream);
 
 /* ksana_sage_attn_fwd restricted by a block mask: block_mask is a device array of int8
@@ -174,10 +182,16 @@ int ksana_sage_attn_fwd(const void* workspace, void* o, int dtype, const int64_t
  * Replaces block_sparse_sage2_attn_cuda(q, k, v, mask_id=..., tensor_layout="NHD")
  * (radial_sage_attn.py:24,170-176: the same mask shape and block sizes); block_mask == NULL is
  * ksana_sage_attn_fwd.  Key tiles neither 128-row half of a 256-row workgroup asks for are skipped. */
-int ksana_sage_attn_fwd_masked(const void* workspace, void* o, int dtype, const int64_t o_strides[4],
+int ksana_sage_attn_fwd_masked(void* workspace, void* o, int dtype, const int64_t o_strides[4],
                                const ksana_sage_shape* shape, const int8_t* block_mask,
                                const int64_t mask_strides[2], const int32_t* k_lens, int causal, int flags,
                                void* stream);
+
+/* How ksana_sage_attn_fwd cuts `shape` on the current device (dense, non-causal calls): the 256-row query blocks
+ * numbered *first_workgroup and up - numbering (b * Hq + h) * ceil(Lq/256) + block - have their key loop cut into
+ * *runs runs; *runs == 0 means no cut.  For tools that want to mirror the kernel's rounding exactly (the test
+ * emulation does); no counterpart in the reference. */
+int ksana_sage_attn_key_split(const ksana_sage_shape* shape, int* first_workgroup, int* runs);
 
 /* The whole path in one call: quant_q, quant_k, quant_v, attn_fwd on `stream`.
  * Replaces sageattn(q, k, v, tensor_layout="NHD", is_causal=causal) (sage_attn.py:75-81). */

@@ -99,15 +99,26 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
   }
 }
 
-template <int DT, bool kPwlExp, bool kSparse>
+// kSplit: the workgroup takes one of `p.n_split` equal runs of key tiles of its (head, query block) and leaves
+// unnormalised accumulators, running maxima and row sums in the workspace for sage_attn_merge_kernel.  Used for
+// the workgroups beyond the last full round of the chip, which would otherwise hold it for a whole round alone.
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit>
 __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg, int n_wg,
                                                                      int wg_per_xcd) {
-  // Consecutive workgroup ids land on consecutive XCDs (8 per chip, one L2 each).  Give every
-  // XCD a contiguous run of (head, query block) pairs so the workgroups that stream the same
-  // K/V tiles share one L2.
-  const int xcd = blockIdx.x & 7;
-  const int wg = xcd * wg_per_xcd + (blockIdx.x >> 3);
-  if (wg >= n_wg) return;
+  static_assert(!(kSparse && kSplit), "the key split is built for the dense loop only");
+  int wg, split = 0;
+  if constexpr (kSplit) {
+    const int item = blockIdx.x / p.n_split;
+    split = blockIdx.x - item * p.n_split;
+    wg = p.split_first_wg + item;
+  } else {
+    // Consecutive workgroup ids land on consecutive XCDs (8 per chip, one L2 each).  Give every
+    // XCD a contiguous run of (head, query block) pairs so the workgroups that stream the same
+    // K/V tiles share one L2.
+    const int xcd = blockIdx.x & 7;
+    wg = xcd * wg_per_xcd + (blockIdx.x >> 3);
+    if (wg >= n_wg) return;
+  }
   const int bh = wg / n_qwg;
   int qwg = wg - bh * n_qwg;
   // causal: the later a query block, the more key tiles it walks - start the long ones first
@@ -132,9 +143,28 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       for (int i = 0; i < 8; ++i) orow[i] = make_uint4(0, 0, 0, 0);
     }
   };
-  if (lk == 0) {
-    write_zero_rows();
-    return;
+  int tile0 = 0;  // first key tile of this workgroup's run
+  if constexpr (kSplit) {
+    const int tiles = (lk + kBlkK - 1) / kBlkK;
+    const int per = (tiles + p.n_split - 1) / p.n_split;
+    tile0 = split * per;
+    const int tile1 = min(tiles, tile0 + per);
+    if (tile0 >= tile1) {  // nothing in this run (few tiles, or a batch entry without keys): an empty partial
+      if (active) {
+        const int row = wave * 32 + l32;
+        float* po = p.split_o + ((int64_t)blockIdx.x * kAttnQPerWg + row) * kD + 64 * hh;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) reinterpret_cast<float4*>(po)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (hh == 0) reinterpret_cast<float2*>(p.split_ml)[(int64_t)blockIdx.x * kAttnQPerWg + row] = make_float2(-INFINITY, 0.f);
+      }
+      return;
+    }
+    lk = min(lk, tile1 * kBlkK) - tile0 * kBlkK;  // from here on the run is the whole key sequence
+  } else {
+    if (lk == 0) {
+      write_zero_rows();
+      return;
+    }
   }
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -184,10 +214,10 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     magic[r] = m;
   }
 
-  const uint8_t* k_src = reinterpret_cast<const uint8_t*>(p.k_tiles) + (int64_t)bhk * p.nkb * kTileBytes;  // uniform
-  const uint8_t* v_src = p.v_tiles + (int64_t)bhk * p.nkb * kTileBytes;
+  const uint8_t* k_src = reinterpret_cast<const uint8_t*>(p.k_tiles) + ((int64_t)bhk * p.nkb + tile0) * kTileBytes;  // uniform
+  const uint8_t* v_src = p.v_tiles + ((int64_t)bhk * p.nkb + tile0) * kTileBytes;
   const unsigned copy_off = tid * 16;  // this lane's 16 bytes inside a tile
-  const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb;
+  const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb + tile0;
   const int nkb = (lk + kBlkK - 1) / kBlkK;  // tiles this batch uses; p.nkb stays the per-head stride
   // K scales live in LDS behind the ring: a per-tile global load would share the in-order
   // vmcnt queue with the tile copies and stall on all of them
@@ -556,6 +586,19 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, lacc, 0, 0, 0, 0, 0, 0);
   }
 
+  if constexpr (kSplit) {
+    // partial result of this run of keys: O^T and the row sum relative to the run's own maximum
+    const int row = wave * 32 + l32;
+    float* po = p.split_o + ((int64_t)blockIdx.x * kAttnQPerWg + row) * kD;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<float4*>(po + 32 * dt + 8 * g + 4 * hh) =
+            make_float4(oacc[dt][4 * g + 0], oacc[dt][4 * g + 1], oacc[dt][4 * g + 2], oacc[dt][4 * g + 3]);
+    if (hh == 0) reinterpret_cast<float2*>(p.split_ml)[(int64_t)blockIdx.x * kAttnQPerWg + row] = make_float2(m_run, lacc[0]);
+    return;
+  }
   // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
   // a mask row that allows none of its keys has an empty sum: its rows are zeros, not 0/0
   const float inv_l = (!kSparse || lacc[0] > 0.0f) ? 1.0f / lacc[0] : 0.0f;
@@ -583,7 +626,42 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   }
 }
 
-template <int DT, bool kPwlExp, bool kSparse>
+// Combines the partial results of the key runs: for every query row the run maxima are brought to a common one,
+// then O = sum_i O_i 2^(m_i - m), l = sum_i l_i 2^(m_i - m), and the usual last step follows.
+// grid = (items, 32), 256 threads: a thread owns one row and four channels of a 8-row slab.
+template <int DT>
+__global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p, int n_qwg) {
+  const int item = blockIdx.x, wg = p.split_first_wg + item;
+  const int bh = wg / n_qwg, qwg = wg - bh * n_qwg;
+  const int b = bh / p.Hq, h = bh - b * p.Hq;
+  const int bhk = b * p.Hkv + h / (p.Hq / p.Hkv);
+  const int row = blockIdx.y * 8 + (threadIdx.x >> 5), d = (threadIdx.x & 31) * 4;
+  const int q = qwg * kAttnQPerWg + row;
+  if (q >= p.Lq) return;
+  const float2* ml = reinterpret_cast<const float2*>(p.split_ml) + (int64_t)item * p.n_split * kAttnQPerWg + row;
+  const float* po = p.split_o + ((int64_t)item * p.n_split * kAttnQPerWg + row) * kD + d;
+  float m = -INFINITY;
+  for (int s = 0; s < p.n_split; ++s) m = fmaxf(m, ml[(int64_t)s * kAttnQPerWg].x);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float l = 0.0f;
+  for (int s = 0; s < p.n_split; ++s) {
+    const float2 e = ml[(int64_t)s * kAttnQPerWg];
+    if (e.y == 0.0f) continue;  // an empty run (its maximum is -inf)
+    const float w = fast_exp2(e.x - m);
+    const float4 o = *reinterpret_cast<const float4*>(po + (int64_t)s * kAttnQPerWg * kD);
+    acc.x += o.x * w, acc.y += o.y * w, acc.z += o.z * w, acc.w += o.w * w;
+    l += e.y * w;
+  }
+  const float inv_l = l > 0.0f ? 1.0f / l : 0.0f;
+  const float keep_mean = l > 0.0f ? 1.0f : 0.0f;
+  const float4 s4 = *reinterpret_cast<const float4*>(p.v_scale + (int64_t)bhk * kD + d);
+  const float4 m4 = *reinterpret_cast<const float4*>(p.v_mean + (int64_t)bhk * kD + d);
+  uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
+  store4<DT>(orow + d, acc.x * inv_l * s4.x + m4.x * keep_mean, acc.y * inv_l * s4.y + m4.y * keep_mean,
+             acc.z * inv_l * s4.z + m4.z * keep_mean, acc.w * inv_l * s4.w + m4.w * keep_mean);
+}
+
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false>
 hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
   // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
@@ -594,18 +672,44 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   if (!requested[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse>),
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             kSparse ? kStages * kStageBytes + 2 * kSparseMaxKeyTiles * 4 + 1024
                                     : kStages * kStageBytes + kMaxKeyTiles * 4);
     if (e != hipSuccess) return e;
     requested[dev].store(true, std::memory_order_release);
   }
-  sage_attn_fwd_kernel<DT, kPwlExp, kSparse><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
 }
 
+// compute units of the current device (the size of one round of workgroups: one workgroup per unit)
+int compute_units() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = cached[dev].load(std::memory_order_acquire);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_release);
+  }
+  return n;
+}
+
 }  // namespace
+
+void plan_key_split(int n_wg, int nkb, int* first_wg, int* runs) {
+  const int cus = compute_units();
+  const int rest = n_wg % cus;
+  int n_split = 0;
+  if (rest != 0 && 2 * rest <= cus) {
+    n_split = min(min(cus / rest, kMaxSplitPartials / rest), nkb / kMinTilesPerSplit);
+    if (n_split < 2) n_split = 0;
+  }
+  *first_wg = n_split ? n_wg - rest : n_wg;
+  *runs = n_split;
+}
 
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   if (p.nkb > kMaxKeyTiles) return hipErrorInvalidValue;
@@ -626,11 +730,42 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   }
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
   const size_t lds = kStages * kStageBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
-  if (p.exact_exp2)
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, false, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
-  return bf16 ? launch_variant<KSANA_SAGE_BF16, true, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
-              : launch_variant<KSANA_SAGE_FP16, true, false>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
+  auto launch_dense = [&](const AttnParams& pp, dim3 g, int wgs, int per_xcd, bool split) -> hipError_t {
+    if (split) {
+      if (pp.exact_exp2)
+        return bf16 ? launch_variant<KSANA_SAGE_BF16, false, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
+                    : launch_variant<KSANA_SAGE_FP16, false, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
+      return bf16 ? launch_variant<KSANA_SAGE_BF16, true, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
+                  : launch_variant<KSANA_SAGE_FP16, true, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
+    }
+    if (pp.exact_exp2)
+      return bf16 ? launch_variant<KSANA_SAGE_BF16, false, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
+                  : launch_variant<KSANA_SAGE_FP16, false, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, true, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, true, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
+  };
+  // The workgroups beyond the last full round of the chip (one workgroup per compute unit) would hold it for a
+  // whole round alone.  When they are few, each is cut into runs of key tiles that together fill a round, and a
+  // small kernel merges the runs: 2568 workgroups are then 10 rounds and a bit instead of 11, 280 are 1.1 instead of 2.
+  int n_full = n_wg, n_split = 0;
+  if (p.split_o != nullptr) plan_key_split(n_wg, p.nkb, &n_full, &n_split);
+  if (n_split == 0) return launch_dense(p, grid, n_wg, wg_per_xcd, false);
+  const int rest = n_wg - n_full;
+  if (n_full > 0) {
+    const int per_xcd = (n_full + 7) / 8;
+    const hipError_t e = launch_dense(p, dim3(per_xcd * 8), n_full, per_xcd, false);
+    if (e != hipSuccess) return e;
+  }
+  AttnParams ps = p;
+  ps.split_first_wg = n_full;
+  ps.n_split = n_split;
+  const hipError_t e = launch_dense(ps, dim3(rest * n_split), n_wg, 0, true);
+  if (e != hipSuccess) return e;
+  if (bf16)
+    sage_attn_merge_kernel<KSANA_SAGE_BF16><<<dim3(rest, kAttnQPerWg / 8), dim3(256), 0, s>>>(ps, n_qwg);
+  else
+    sage_attn_merge_kernel<KSANA_SAGE_FP16><<<dim3(rest, kAttnQPerWg / 8), dim3(256), 0, s>>>(ps, n_qwg);
+  return hipGetLastError();
 }
 
 }  // namespace ksana_sage

@@ -183,6 +183,8 @@ int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout*
   l.q_rms = take((uint64_t)s->B * s->Lq * 4);
   l.k_rms = take((uint64_t)s->B * s->Lk * 4);
   l.v_mean = take(bhk * kD * 4);
+  l.split_o = take((uint64_t)kMaxSplitPartials * kAttnQPerWg * kD * 4);
+  l.split_ml = take((uint64_t)kMaxSplitPartials * kAttnQPerWg * 2 * 4);
   l.total_bytes = off;
   *out = l;
   return 0;
@@ -293,12 +295,21 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], con
   return e == hipSuccess ? 0 : hip_fail(e, "quant_v launch");
 }
 
-int ksana_sage_attn_fwd(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
+int ksana_sage_attn_key_split(const ksana_sage_shape* s, int* first_workgroup, int* runs) {
+  if (int rc = check_shape(s)) return rc;
+  if (!first_workgroup || !runs) return fail(KSANA_SAGE_EINVAL, "out-pointer is null");
+  const int n_qwg = (s->Lq + ksana_sage::kAttnQPerWg - 1) / ksana_sage::kAttnQPerWg;
+  ksana_sage::plan_key_split(s->B * s->Hq * n_qwg, (s->Lk + ksana_sage::kBlkK - 1) / ksana_sage::kBlkK, first_workgroup,
+                             runs);
+  return 0;
+}
+
+int ksana_sage_attn_fwd(void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
                         const int32_t* k_lens, int causal, int flags, void* stream) {
   return ksana_sage_attn_fwd_masked(ws, o, dtype, o_st, s, nullptr, nullptr, k_lens, causal, flags, stream);
 }
 
-int ksana_sage_attn_fwd_masked(const void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
+int ksana_sage_attn_fwd_masked(void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
                                const int8_t* block_mask, const int64_t mask_st[2], const int32_t* k_lens, int causal,
                                int flags, void* stream) {
   if (int rc = check_shape(s)) return rc;
@@ -318,6 +329,9 @@ int ksana_sage_attn_fwd_masked(const void* ws, void* o, int dtype, const int64_t
   p.v_tiles = ws_at<uint8_t>(ws, l.v_fp8);
   p.v_scale = ws_at<float>(ws, l.v_scale);
   p.v_mean = ws_at<float>(ws, l.v_mean);
+  p.split_o = ws_at<float>(ws, l.split_o);
+  p.split_ml = ws_at<float>(ws, l.split_ml);
+  p.split_first_wg = 0, p.n_split = 0;
   p.o = ksana_sage::OutTensor{static_cast<uint16_t*>(o), o_st[0], o_st[1], o_st[2], dtype};
   p.B = s->B, p.Hq = s->Hq, p.Hkv = s->Hkv, p.Lq = s->Lq, p.Lk = s->Lk;
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;

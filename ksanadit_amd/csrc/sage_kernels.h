@@ -81,9 +81,19 @@ struct AttnParams {
   const int8_t* block_mask;
   int64_t mask_sB, mask_sH;  // element strides of the two leading dims (0 broadcasts)
   int causal;  // 1: query row i attends to keys [0, i] only (on top of k_lens and the block mask)
+  // scratch for workgroups cut into runs of key tiles (nullptr: never cut): per partial 256 rows x 128 fp32
+  // accumulators, and per row its running maximum and row sum; room for kMaxSplitPartials partials
+  float* split_o;
+  float* split_ml;
+  int split_first_wg, n_split;  // filled in by the launcher
 };
+constexpr int kMaxSplitPartials = 256;  // (workgroups beyond the last full round) x (runs each) never exceeds this
+constexpr int kMinTilesPerSplit = 8;    // a run shorter than this does not repay its prologue
 constexpr int kMaskBlkQ = 128;           // query rows per mask row (two per workgroup)
 constexpr int kSparseMaxKeyTiles = 2048; // key tiles per head with a block mask or causal masking (tile list lives in LDS)
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s);
+// Which of `n_wg` dense workgroups the launcher cuts into runs of key tiles on the current device, and into how
+// many: workgroups [*first_wg, n_wg) into *runs each; *runs == 0 means none.
+void plan_key_split(int n_wg, int nkb, int* first_wg, int* runs);
 
 }  // namespace ksana_sage

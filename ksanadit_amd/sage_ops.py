@@ -257,6 +257,15 @@ def _block_mask_arg(block_mask, B: int, H: int, Lq: int, Lk: int, device):
     return m, strides
 
 
+def key_split_plan(ws: SageWorkspace):
+    """``(first_workgroup, runs)`` of the cut the dense, non-causal attention call makes for this workspace's shape on
+    the current device, or ``None`` when it makes none (see ``ksana_sage_attn_key_split``)."""
+    first, runs = C.c_int(0), C.c_int(0)
+    _capi.check(_capi.load().ksana_sage_attn_key_split(C.byref(ws.shape), C.byref(first), C.byref(runs)),
+                "ksana_sage_attn_key_split")
+    return (first.value, runs.value) if runs.value else None
+
+
 def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False,
              k_lens=None, block_mask=None) -> torch.Tensor:
     """Attention on the quantized operands in ``ws``.  ``k_lens`` (optional, one int per batch entry): batch ``b``

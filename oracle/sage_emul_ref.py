@@ -42,7 +42,7 @@ def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
 
 
 def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True,
-                         exact_exp2=True, k_lens=None, block_mask=None, v_mean=None):
+                         exact_exp2=True, k_lens=None, block_mask=None, v_mean=None, key_split=None):
     """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
 
     ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
@@ -53,6 +53,10 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     with a non-zero entry ``(i, j)``; rows without any tile give zeros (online form only).
     ``v_mean`` (``[B, Hkv, D]``, optional): the channel mean the V quantizer took off (``quant_v_ref(..., smooth_v=True)``);
     it is added back to every output row that saw at least one key.
+    ``key_split`` (``(first_workgroup, runs)``, optional, dense online form only): the kernel cuts the key loop of
+    the 256-row query blocks numbered ``first_workgroup`` and up (numbering: ``(b * H + h) * ceil(Lq/256) + block``)
+    into ``runs`` equal runs of key tiles, walks each run on its own and merges the partial results; probabilities are
+    then rounded relative to the run's own running maximum, which this mirrors.
     ``causal`` (``Lq == Lk`` only): row ``i`` sees keys ``[0, i]``; in the online form a row sits out the tiles that
     start after it and sees a prefix of the tile that holds its own position.
     """
@@ -95,12 +99,18 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 #   exponent = fma(x_f, sc, c)          (pwl: fma(x_f, 8 sc, fma(8, c, 55.5)))
                 magic = 12582912.0
                 x_f = (s_int + magic).to(torch.float32)  # exact: |dot| < 2**22
-                m = torch.full((Lq, 1), float("-inf"))
-                l = torch.zeros(Lq, 1)
-                acc = torch.zeros(Lq, D)
                 rows = torch.arange(Lq)[:, None]
-                for j0 in range(0, lk_b, BLKK):
-                    j1 = min(j0 + BLKK, lk_b)
+
+                def walk(key_from, key_to):
+                    """Online softmax over the tiles of keys [key_from, key_to): (acc, m, l)."""
+                    m = torch.full((Lq, 1), float("-inf"))
+                    l = torch.zeros(Lq, 1)
+                    acc = torch.zeros(Lq, D)
+                    for j0 in range(key_from, key_to, BLKK):
+                        m, l, acc = step(j0, min(j0 + BLKK, key_to), m, l, acc)
+                    return acc, m, l
+
+                def step(j0, j1, m, l, acc):
                     act = None  # rows that take part in this step
                     if block_mask is not None:
                         # rows of a 128-row block that does not ask for this tile sit the step out
@@ -112,7 +122,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                         allow = torch.arange(j0, j1)[None, :] <= rows
                         act = allow[:, :1] if act is None else (act & allow[:, :1])
                     if act is not None and not bool(act.any()):
-                        continue
+                        return m, l, acc
                     sc = (qs_row[b, h][:, None] * k_scale[b, hk, j0 // BLKK]).to(torch.float32)
                     xt = x_f[:, j0:j1]
                     mneg = -(magic * sc)  # fp32
@@ -138,7 +148,23 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                         p8 = torch.where(act, p8, torch.zeros_like(p8))
                     l = l * alpha + p8.sum(dim=1, keepdim=True)  # the normaliser sees the rounded P too
                     acc = acc * alpha + p8 @ vf[j0:j1]
-                    m = m_new
+                    return m_new, l, acc
+
+                acc, m, l = walk(0, lk_b)
+                if key_split is not None:
+                    if causal or block_mask is not None:
+                        raise NotImplementedError("key_split with causal masking or a block mask")
+                    first_wg, runs = key_split
+                    n_qwg = (Lq + 255) // 256
+                    tiles = (lk_b + BLKK - 1) // BLKK
+                    per = (tiles + runs - 1) // runs
+                    parts = [walk(r * per * BLKK, min(lk_b, (r + 1) * per * BLKK)) for r in range(runs) if r * per < tiles]
+                    m_all = torch.stack([pm for _, pm, _ in parts]).amax(dim=0)
+                    acc_s = sum(pa * torch.exp2(pm - m_all) for pa, pm, _ in parts)
+                    l_s = sum(pl * torch.exp2(pm - m_all) for _, pm, pl in parts)
+                    wg_of_row = (b * H + h) * n_qwg + torch.arange(Lq) // 256
+                    cut = (wg_of_row >= first_wg)[:, None]
+                    acc, l = torch.where(cut, acc_s, acc), torch.where(cut, l_s, l)
                 o = acc / l * v_scale[b, hk][None, :]
                 if v_mean is not None:
                     o = o + v_mean[b, hk].float()[None, :]

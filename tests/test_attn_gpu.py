@@ -30,11 +30,13 @@ def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
 
 
 def _emul_from_ws(ws, Lq, Lk, dtype, exact_exp2=True, k_lens=None, block_mask=None, causal=False):
-    """The CPU emulation fed with the operands the GPU quantizer actually produced."""
+    """The CPU emulation fed with the operands the GPU quantizer actually produced, and cut into the same runs of key
+    tiles as the kernel cuts the query blocks beyond its last full round (dense, non-causal calls)."""
+    split = None if (causal or block_mask is not None) else sage_ops.key_split_plan(ws)
     return sage_emul_from_quant(
         ws.q_i8.cpu()[:, :, :Lq], ws.q_scale.cpu()[:, :, :Lq], untile_k(ws.k_tiles.cpu(), Lk), ws.k_scale.cpu(),
         untile_v(ws.v_tiles.cpu(), Lk).view(torch.float8_e4m3fn), ws.v_scale.cpu(), dtype, exact_exp2=exact_exp2,
-        k_lens=k_lens, block_mask=block_mask, causal=causal,
+        k_lens=k_lens, block_mask=block_mask, causal=causal, key_split=split,
     )
 
 
@@ -199,10 +201,14 @@ def test_block_mask_limits_query_blocks_to_key_tiles(hip_device, B, Lq, Lk, H, d
     assert (out[0, 128 * (nq - 1):, 0] == 0).all() and (ref[0, 128 * (nq - 1):, 0] == 0).all()
     assert _cos(out, ref) >= (COS_MIN if exact else 0.9985)
     assert (out.float() - ref.float()).abs().max() <= 0.12 * max(ref.float().abs().max().item(), 0.1)
-    # an all-ones mask is the dense kernel's result, bit for bit; a [nq, nk] mask broadcasts
+    # an all-ones mask is the dense kernel's result (bit for bit when the dense call walks its keys in one run); a
+    # [nq, nk] mask broadcasts
     dense = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact).cpu()
     ones = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact, block_mask=torch.ones(nq, nk)).cpu()
-    assert torch.equal(dense, ones)
+    if sage_ops.key_split_plan(ws) is None:
+        assert torch.equal(dense, ones)
+    else:  # the dense call cuts its key loop into runs on a grid this small: same attention, other rounding points
+        assert _cos(dense, ones) > 0.999
     # tiles no row asks for never reach the result: overwrite their quantized images and rerun
     unused = (mask.view(B, H, -1, nk).sum(dim=2) == 0)  # [B, H, nk]
     before = sage_ops.attn_fwd(ws, torch.empty_like(qd), pwl_exp2=not exact, block_mask=mask).cpu()
@@ -446,6 +452,45 @@ def test_v_smoothing_adds_the_mean_back(hip_device, exact):
     assert torch.equal(impl.forward(qd, kd, vd).cpu(), out)
     half = sage_ops.sageattn(qd, kd, vd, smooth_v=True, pwl_exp2=not exact, out_dtype=torch.float16).cpu()
     assert (half.float() - out.float()).abs().max() <= 2.0**-7 * out.float().abs().max()
+
+
+@pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
+@pytest.mark.parametrize("B,Lq,Lk,Hq,Hkv,dtype,k_lens", [
+    (1, 100, 1000, 2, 2, torch.bfloat16, None),      # 2 query blocks, 16 key tiles -> 2 runs each
+    (1, 300, 2100, 3, 1, torch.float16, None),       # 6 blocks, ragged last tile, grouped heads
+    (2, 700, 4096, 2, 2, torch.bfloat16, [4096, 1500]),  # per-batch key counts: later runs of batch 1 are empty
+    (1, 256, 8192, 1, 1, torch.bfloat16, [0]),       # no keys at all: every run empty, zeros out
+])
+def test_key_loop_cut_into_runs_for_small_grids(hip_device, B, Lq, Lk, Hq, Hkv, dtype, k_lens, exact):
+    """Grids that leave most of the chip idle: the kernel cuts each query block's key loop into runs and merges.
+    Against the emulation cut the same way (tight), SDPA, the uncut result of the tile-list kernel under an all-ones
+    mask, and itself (identical bits on a second call)."""
+    print(f"case split B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv} {dtype} k_lens={k_lens} exact={exact}", flush=True)
+    q, k, v = _rand_qkv(B, Lq, Lk, Hq, Hkv, seed=Lq + Lk, dtype=dtype)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    plan = sage_ops.key_split_plan(ws)
+    assert plan is not None and plan[0] == 0 and plan[1] >= 2, plan
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, k_lens=k_lens, pwl_exp2=not exact)
+    again = sage_ops.attn_fwd(ws, torch.empty_like(qd), k_lens=k_lens, pwl_exp2=not exact)
+    assert torch.equal(out, again)
+    out = out.cpu()
+    assert torch.isfinite(out.float()).all()
+    emul = _emul_from_ws(ws, Lq, Lk, dtype, exact, k_lens=k_lens)
+    scale = max(emul.float().abs().max().item(), 1e-3)
+    diff = (out.float() - emul.float()).abs()
+    assert diff.max() <= 2e-2 * scale
+    assert (diff > 1e-2 * scale * 0.5).float().mean() <= 1e-3
+    ref = sdpa_ref(q, k, v, k_lens=k_lens)
+    if k_lens != [0]:
+        assert _cos(out, ref) >= (COS_MIN if exact else 0.9985)
+    else:
+        assert (out == 0).all() and (ref == 0).all()
+    uncut = sage_ops.attn_fwd(ws, torch.empty_like(qd), k_lens=k_lens, pwl_exp2=not exact,
+                              block_mask=torch.ones(-(-Lq // 128), -(-Lk // 64))).cpu()
+    assert (out.float() - uncut.float()).abs().max() <= 0.08 * max(uncut.float().abs().max().item(), 1e-3)
+    if k_lens != [0]:
+        assert _cos(out, uncut) > 0.999
 
 
 def test_backend_k_lens_is_opt_in(hip_device):

@@ -48,7 +48,9 @@ def test_workspace_layout_headline_shape():
     assert offs == sorted(offs) and all(o % 256 == 0 for o in offs) and lay.total_bytes % 256 == 0
     assert lay.q_scale - lay.q_i8 == w.H * 32768 * 128  # int8 Q, padded to 128 rows
     assert lay.k_scale - lay.k_i8 == w.H * 512 * TILE_BYTES
-    assert lay.total_bytes < 3 * w.elements + (16 << 20)  # three 8-bit tensors, scales, partial sums
+    # three 8-bit tensors, scales, partial sums, and the fixed 34 MB scratch of the key-split workgroups
+    assert lay.total_bytes < 3 * w.elements + (52 << 20)
+    assert lay.split_ml - lay.split_o == 256 * 256 * 128 * 4
 
 
 @pytest.mark.parametrize(

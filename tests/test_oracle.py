@@ -471,6 +471,44 @@ def test_sage_emul_causal_equals_emulating_each_row_on_its_prefix():
     assert _cos(sdpa_ref(q, k, v, causal=True), ref) > 0.999
 
 
+def test_sage_emul_key_split_merges_runs_of_keys():
+    """key_split: the query blocks from a given number on walk their keys in equal runs of tiles and merge.  Pinned
+    by (a) one run == no split, bit for bit; (b) only the blocks from that number on change; (c) an independent
+    merge: each run emulated alone on the cut operands, combined with the exact softmax mass of its keys from a
+    float64 computation on the same quantized operands."""
+    B, Lq, Lk, H, D = 1, 300, 1100, 2, 128
+    q, k, v = _rand((B, Lq, H, D), 81), _rand((B, Lk, H, D), 82), _rand((B, Lk, H, D), 83)
+    q_i8, q_s = qr.quant_q_ref(q, D**-0.5)
+    k_i8, k_s, _ = qr.quant_k_ref(k)
+    v_f8, v_s = qr.quant_v_ref(v)
+    emul = lambda **kw: sage_emul_from_quant(q_i8, q_s, k_i8, k_s, v_f8, v_s, torch.bfloat16, **kw)  # noqa: E731
+    plain = emul()
+    assert torch.equal(emul(key_split=(0, 1)), plain)
+    runs = 3
+    cut = emul(key_split=(1, runs))  # blocks: head 0 -> 0, 1; head 1 -> 2, 3; block 0 stays whole
+    assert torch.equal(cut[:, :256, 0], plain[:, :256, 0])
+    assert not torch.equal(cut[:, 256:, 0], plain[:, 256:, 0]) and not torch.equal(cut[:, :, 1], plain[:, :, 1])
+    assert _cos(cut, plain) > 0.9995  # same attention, P rounded relative to other maxima
+    # independent merge for head 1: tiles 18 -> runs of 6 tiles = 384 keys
+    per = 6 * 64
+    s = (q_i8[0, 1].double() * q_s[0, 1].double()[:, None]) @ (k_i8[0, 1].double() * k_s[0, 1].double().repeat_interleave(64)[:Lk, None]).t()
+    mass = torch.stack([torch.exp2(s[:, r * per : (r + 1) * per] - s.amax(dim=1, keepdim=True)).sum(dim=1) for r in range(runs)])
+    weight = mass / mass.sum(dim=0, keepdim=True)  # [runs, Lq]
+    want = torch.zeros(Lq, D, dtype=torch.float64)
+    for r in range(runs):
+        lo, hi = r * per, min(Lk, (r + 1) * per)
+        alone = sage_emul_from_quant(q_i8[:, 1:2], q_s[:, 1:2], k_i8[:, 1:2, lo:hi], k_s[:, 1:2, lo // 64 : (hi + 63) // 64],
+                                     v_f8[:, 1:2, lo:hi], v_s[:, 1:2], torch.float32)
+        want += weight[r][:, None] * alone[0, :, 0].double()
+    got = cut[0, :, 1].double()
+    assert (got - want).abs().max() < 6e-3 * want.abs().max() + 2e-3  # bf16 output, row sums from rounded P
+    # with per-batch key counts the runs are cut from the keys that count
+    lens = [700]
+    a = emul(key_split=(0, 2), k_lens=lens)
+    b = sage_emul_from_quant(q_i8, q_s, k_i8[:, :, :700], k_s[:, :, :11], v_f8[:, :, :700], v_s, torch.bfloat16, key_split=(0, 2))
+    assert torch.equal(a, b)
+
+
 # ------------------------------------------------------------------ emulation of the fused kernel
 def _cos(a, b):
     a, b = a.double().flatten(), b.double().flatten()
