@@ -537,6 +537,10 @@ def test_full_size_properties(hip_device, name):
     w = WORKLOADS[name]
     q, k, v = make_inputs(w, device=hip_device)
     out = sage_ops.sageattn(q, k, v)
+    if name == "wan14b_480p":  # 5 120 workgroups are 20 full rounds of the 256 compute units: nothing to cut
+        assert sage_ops.key_split_plan(sage_ops.workspace_for(q, k)) is None
+    if name == "wan5b_720p":  # 2 568 = 10 rounds + 8: those 8 are cut into 32 runs each
+        assert sage_ops.key_split_plan(sage_ops.workspace_for(q, k)) == (2560, 32)
     sdpa = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.TORCH_SDPA))(num_heads=w.H, head_size=w.D)
     c_min, worst = 1.0, 0.0
     for h0 in range(0, w.H, 8):  # by head groups: keeps the fp64 reductions small
