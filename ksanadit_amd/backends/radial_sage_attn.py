@@ -36,7 +36,7 @@ class RadialSageAttentionImpl(KsanaAttentionBackendImpl):
 
     @staticmethod
     def supports(**kwargs) -> bool:
-        if not platform.is_gpu():
+        if not platform.is_sage_device():
             return False
         _capi.load()
         head_size = kwargs.get("head_size")

@@ -43,7 +43,7 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
 
     @staticmethod
     def supports(**kwargs) -> bool:
-        if not platform.is_gpu():
+        if not platform.is_sage_device():
             return False
         _capi.load()  # raises SageLibraryError on a GPU host whose library is missing or stale
         head_size = kwargs.get("head_size")

@@ -57,7 +57,7 @@ __device__ __forceinline__ void lds_copy16(const void* gbase, unsigned lane_off,
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_off), "v"(lane_off), "s"(gbase)
-               : "memory");
+               : "memory", "m0");
 }
 
 // Opaque use+def at this program point: keeps the optimizer from sinking the computation of

@@ -33,6 +33,12 @@ int check_shape(const ksana_sage_shape* s) {
   if (s->Lk > 262144) return fail(KSANA_SAGE_ENOTSUP, "Lk=%d exceeds 262144 (K scales of one head are kept in LDS)", s->Lk);
   if ((int64_t)s->B * s->Hq > 65535 * 8 || s->Hq > 65535 || s->B > 65535)
     return fail(KSANA_SAGE_EINVAL, "B*H too large for the launch grid");
+  // row numbers go through fp32 in the rotary step (exact below 2^24), and the kernels index workgroups with int32
+  if (s->Lq > (1 << 24)) return fail(KSANA_SAGE_ENOTSUP, "Lq=%d exceeds %d", s->Lq, 1 << 24);
+  const int64_t n_wg = (int64_t)s->B * s->Hq * ((s->Lq + ksana_sage::kAttnQPerWg - 1) / ksana_sage::kAttnQPerWg);
+  if (n_wg > (INT64_C(1) << 31) / 8 - 8)
+    return fail(KSANA_SAGE_ENOTSUP, "B*Hq*ceil(Lq/256) = %lld workgroups exceed the launch grid (%lld)",
+                (long long)n_wg, (long long)((INT64_C(1) << 31) / 8 - 8));
   return 0;
 }
 

@@ -27,3 +27,13 @@ def gcn_arch(index: int = 0) -> str:
     if not is_gpu():
         return ""
     return torch.cuda.get_device_properties(index).gcnArchName.split(":")[0]
+
+
+SAGE_ARCH = "gfx950"  # the only architecture libksana_sage_hip.so holds code for
+
+
+def is_sage_device() -> bool:
+    """True when the HIP library's kernels can run here: a HIP device of the architecture it was compiled for.
+    On any other device the selector moves on to the next backend, as the reference's availability probe makes it
+    (ksana/operations/attention/backends/sage_attn.py:21-27,36-38), instead of failing at the first launch."""
+    return gcn_arch() == SAGE_ARCH

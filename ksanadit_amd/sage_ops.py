@@ -19,6 +19,7 @@ import torch
 
 from . import _capi
 from .layout import TILE_BYTES
+from .logger import log
 
 _DTYPES = {torch.bfloat16: _capi.BF16, torch.float16: _capi.FP16}
 
@@ -27,12 +28,22 @@ def _strides(t: torch.Tensor):
     return _capi.Strides(*t.stride())
 
 
+_copy_warned = False
+
+
 def _usable(t: torch.Tensor) -> torch.Tensor:
-    """The kernels read 16 bytes at a time along D: fix up layouts that do not allow it."""
+    """The kernels read 16 bytes at a time along D: fix up layouts that do not allow it.  The fix-up is a full
+    copy of the tensor (one more read and write of it ahead of an HBM-bound stage), so the first one is logged."""
+    global _copy_warned
     s = t.stride()
     ok = s[3] == 1 and all(x % 8 == 0 and x > 0 for x, n in zip(s[:3], t.shape[:3]) if n > 1)
     if ok and t.data_ptr() % 16 == 0:
         return t
+    if not _copy_warned:
+        _copy_warned = True
+        log.warning("Sage HIP path: copying a tensor of shape %s, strides %s (the kernels need a unit D stride, other "
+                    "strides multiples of 8 and a 16-byte aligned base); further copies are not logged",
+                    tuple(t.shape), tuple(s))
     return t.contiguous()
 
 
@@ -72,6 +83,22 @@ class SageWorkspace:
     @property
     def ptr(self) -> C.c_void_p:
         return C.c_void_p(self.blob.data_ptr())
+
+    def require(self, device, *, B=None, Hq=None, Hkv=None, Lq=None, Lk=None, D=None) -> None:
+        """Refuse a workspace laid out for other extents than the tensors about to be handed to the library: it
+        takes B/H/L from the workspace's shape but pointers and strides from the tensors, so a mismatch would read
+        and write out of bounds.  ``None`` extents are not checked (a stage that sees only q knows nothing of Lk)."""
+        s = self.shape
+        want = {"B": B, "Hq": Hq, "Hkv": Hkv, "Lq": Lq, "Lk": Lk, "D": D}
+        bad = {n: (getattr(s, n), x) for n, x in want.items() if x is not None and getattr(s, n) != x}
+        if bad:
+            detail = ", ".join(f"{n}: workspace {a}, tensor {b}" for n, (a, b) in bad.items())
+            raise ValueError(f"workspace was laid out for another shape ({detail})")
+        if self.blob.device != torch.device(device):
+            raise ValueError(f"workspace lives on {self.blob.device}, the tensors on {device}")
+        if self.blob.dtype != torch.uint8 or self.blob.numel() < self.layout.total_bytes:
+            raise ValueError(f"workspace blob holds {self.blob.numel() * self.blob.element_size()} bytes, "
+                             f"the layout needs {self.layout.total_bytes}")
 
     def _view(self, off: int, nbytes: int, dtype, shape):
         return self.blob[off : off + nbytes].view(dtype).view(shape)
@@ -190,6 +217,7 @@ def workspace_for(q: torch.Tensor, k: torch.Tensor) -> SageWorkspace:
 
 def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: WanPrep | None = None) -> None:
     _require_hip(q)
+    ws.require(q.device, B=q.shape[0], Lq=q.shape[1], Hq=q.shape[2], D=q.shape[3])
     q = _usable(q)
     lib = _capi.load()
     if prep is None:
@@ -204,6 +232,7 @@ def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: WanPrep |
 
 def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: WanPrep | None = None) -> None:
     _require_hip(k)
+    ws.require(k.device, B=k.shape[0], Lk=k.shape[1], Hkv=k.shape[2], D=k.shape[3])
     k = _usable(k)
     lib = _capi.load()
     if prep is None:
@@ -219,6 +248,7 @@ def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: Wan
 def quant_v(v: torch.Tensor, ws: SageWorkspace, smooth_v: bool = False) -> None:
     """``smooth_v``: take the channel means off before scaling; the attention adds them back to its output."""
     _require_hip(v)
+    ws.require(v.device, B=v.shape[0], Lk=v.shape[1], Hkv=v.shape[2], D=v.shape[3])
     v = _usable(v)
     lib = _capi.load()
     rc = lib.ksana_sage_quant_v_smooth(v.data_ptr(), _DTYPES[v.dtype], _strides(v), C.byref(ws.shape), int(smooth_v),
@@ -275,6 +305,9 @@ def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp
     ``128 i ..`` attend to keys ``64 j ..`` - the ``mask_id`` of the reference's block-sparse call
     (radial_sage_attn.py:170-176)."""
     _require_hip(out)
+    if out.dim() != 4:
+        raise ValueError("out must be [B, Lq, H, D]")
+    ws.require(out.device, B=out.shape[0], Lq=out.shape[1], Hq=out.shape[2], D=out.shape[3])
     lib = _capi.load()
     flags = _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0
     kl = _k_lens_arg(k_lens, out.shape[0], out.device)
@@ -337,6 +370,7 @@ def sageattn(
         return out.transpose(1, 2) if tensor_layout == "HND" else out
     sm_scale = D**-0.5 if sm_scale is None else float(sm_scale)
     ws = workspace_for(q, k) if workspace is None else workspace
+    ws.require(q.device, B=B, Hq=Hq, Hkv=k.shape[2], Lq=Lq, Lk=k.shape[1], D=D)
     out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)

@@ -56,11 +56,44 @@ def test_workspace_layout_headline_shape():
 @pytest.mark.parametrize(
     "args,exc",
     [((1, 4, 4, 16, 16, 64), NotImplementedError), ((1, 4, 3, 16, 16, 128), ValueError), ((1, 4, 4, 0, 16, 128), ValueError),
-     ((0, 4, 4, 16, 16, 128), ValueError), ((1, 4, 4, 16, 262145, 128), NotImplementedError), ((1, 70000, 70000, 16, 16, 128), ValueError)],
+     ((0, 4, 4, 16, 16, 128), ValueError), ((1, 4, 4, 16, 262145, 128), NotImplementedError), ((1, 70000, 70000, 16, 16, 128), ValueError),
+     ((1, 4, 4, (1 << 24) + 1, 16, 128), NotImplementedError), ((8, 65535, 65535, 1 << 20, 16, 128), NotImplementedError)],
 )
 def test_workspace_layout_rejects_bad_shapes(args, exc):
     with pytest.raises(exc):
         _capi.workspace_layout(*args)
+
+
+def test_a_workspace_for_another_shape_is_refused_before_any_launch():
+    """The library takes B/H/L from the workspace's shape and pointers/strides from the tensors: a workspace laid out
+    for other extents (say one reused across self- and cross-attention) must never reach it."""
+    shape, layout = _capi.workspace_layout(1, 4, 4, 512, 512, 128)
+    ws = sage_ops.SageWorkspace(shape, layout, torch.empty(layout.total_bytes, dtype=torch.uint8))
+    ws.require("cpu", B=1, Hq=4, Hkv=4, Lq=512, Lk=512, D=128)
+    ws.require("cpu", B=1, Lq=512)  # a stage that knows only some extents
+    with pytest.raises(ValueError, match="Lk: workspace 512, tensor 77"):
+        ws.require("cpu", B=1, Hq=4, Hkv=4, Lq=512, Lk=77, D=128)
+    with pytest.raises(ValueError, match="another shape"):
+        ws.require("cpu", B=2, Lq=512)
+    with pytest.raises(ValueError, match="lives on"):
+        ws.require("meta", B=1)
+    short = sage_ops.SageWorkspace(shape, layout, torch.empty(layout.total_bytes - 256, dtype=torch.uint8))
+    with pytest.raises(ValueError, match="the layout needs"):
+        short.require("cpu", B=1)
+
+
+def test_sage_backends_need_the_architecture_the_library_was_built_for(monkeypatch):
+    """On a HIP device of another architecture the selector must move on (no code object would load)."""
+    from ksanadit_amd import platform
+    from ksanadit_amd.backends.radial_sage_attn import RadialSageAttentionImpl
+    from ksanadit_amd.backends.sage_sla import SageSLAAttentionImpl
+
+    monkeypatch.setattr(platform, "gcn_arch", lambda index=0: "gfx942")
+    for impl in (SageAttentionImpl, RadialSageAttentionImpl, SageSLAAttentionImpl):
+        assert impl.supports(head_size=128, dtype=torch.bfloat16) is False
+    monkeypatch.setattr(platform, "gcn_arch", lambda index=0: "gfx950")
+    assert SageAttentionImpl.supports(head_size=128, dtype=torch.bfloat16) is True
+    assert SageAttentionImpl.supports(head_size=96, dtype=torch.bfloat16) is False
 
 
 def test_entry_points_validate_before_touching_the_gpu():
