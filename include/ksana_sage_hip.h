@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 7
+#define KSANA_SAGE_ABI_VERSION 8
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -130,6 +130,16 @@ int ksana_sage_quant_q(const void* q, int dtype, const int64_t q_strides[4], con
  * (K half of sage_sla.py:202-204). */
 int ksana_sage_quant_k(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
                        int smooth_k, void* workspace, void* stream);
+
+/* ksana_sage_quant_k for callers that cannot allocate device memory - code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it - and therefore cannot grow a workspace for a new shape's scratch.  No counterpart
+ * in the reference.  Same arguments, same results bit for bit; the difference is where the kernels' scratch (the
+ * per-256-row chunk sums behind the channel means) lives: not in the workspace's k_part area, which this call
+ * leaves untouched, but in an 8 MiB array inside the library's own device image.  Limit: B * Hkv * ceil(Lk / 256)
+ * <= 16384 (KSANA_SAGE_ENOTSUP beyond).  The call allocates and frees nothing.  All calls on one GPU share that
+ * array: calls that overlap on one GPU (different streams or threads) race and must be ordered by the caller. */
+int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
+                              int smooth_k, void* workspace, void* stream);
 
 /* quant_q / quant_k with the step before attention folded in: q and k are the projections
  * viewed [B, L, H, D] (the H stride must be D: a token row is one contiguous run of H*D channels).

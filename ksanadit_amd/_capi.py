@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -24,6 +24,7 @@ EXPORTS = (
     "ksana_sage_workspace_layout",
     "ksana_sage_quant_q",
     "ksana_sage_quant_k",
+    "ksana_sage_quant_k_static",
     "ksana_sage_quant_v",
     "ksana_sage_quant_v_smooth",
     "ksana_sage_attn_fwd",
@@ -81,6 +82,7 @@ def _declare(lib):
     lib.ksana_sage_workspace_layout.argtypes, lib.ksana_sage_workspace_layout.restype = [sp, lp], i
     lib.ksana_sage_quant_q.argtypes, lib.ksana_sage_quant_q.restype = [vp, i, st, sp, f, vp, vp], i
     lib.ksana_sage_quant_k.argtypes, lib.ksana_sage_quant_k.restype = [vp, i, st, sp, i, vp, vp], i
+    lib.ksana_sage_quant_k_static.argtypes, lib.ksana_sage_quant_k_static.restype = [vp, i, st, sp, i, vp, vp], i
     lib.ksana_sage_quant_v.argtypes, lib.ksana_sage_quant_v.restype = [vp, i, st, sp, vp, vp], i
     lib.ksana_sage_quant_v_smooth.argtypes, lib.ksana_sage_quant_v_smooth.restype = [vp, i, st, sp, i, vp, vp], i
     lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, vp, i, i, vp], i

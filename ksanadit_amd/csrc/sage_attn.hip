@@ -52,6 +52,10 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // ALL outstanding LDS reads before every use (lgkmcnt(0)), which serialises the operand
 // prefetch.  The copy is tracked by hand instead (vmcnt, see tile_barrier).
 // The global address is a wave-uniform base (scalar registers) plus a 32-bit per-lane offset.
+// M0 is written and named as clobbered; the compiler remarks that M0 is a register it reserves (it re-materialises
+// M0 before each of its own uses and never keeps a value live in it), which is the behaviour relied on here.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void lds_copy16(const void* gbase, unsigned lane_off, const void* lds_dst) {
   const unsigned lds_off = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)lds_dst;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -59,6 +63,7 @@ __device__ __forceinline__ void lds_copy16(const void* gbase, unsigned lane_off,
                : "s"(lds_off), "v"(lane_off), "s"(gbase)
                : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // Opaque use+def at this program point: keeps the optimizer from sinking the computation of
 // `x` into a later basic block (it emits no instruction).

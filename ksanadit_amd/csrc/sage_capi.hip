@@ -5,9 +5,17 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/ksana_sage_hip.h"
 #include "sage_kernels.h"
+
+// Scratch of ksana_sage_quant_k_static: the chunk sums of K's channel means, [B * Hkv * ceil(Lk / 256)][128]
+// fp32.  Device memory that belongs to the loaded code object: every GPU the library runs on holds its own copy
+// (8 MiB) at its own address from the first launch on it until the process ends.  In host code the name below is
+// only a handle for hipGetSymbolAddress - the device address it yields is what kernels are given.
+constexpr int kStaticChunkRows = 16384;  // B * Hkv * ceil(Lk / 256) that fit
+static __device__ __align__(256) float scratch[(size_t)kStaticChunkRows * ksana_sage::kD];
 
 namespace {
 
@@ -72,6 +80,28 @@ T* ws_at(void* ws, uint64_t off) {
 template <typename T>
 const T* ws_at(const void* ws, uint64_t off) {
   return reinterpret_cast<const T*>(static_cast<const uint8_t*>(ws) + off);
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(float** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(KSANA_SAGE_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(KSANA_SAGE_ENOTSUP, "device index %d beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(KSANA_SAGE_EHIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
 }
 
 int check_ws(const void* ws) {
@@ -232,8 +262,9 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
   return ksana_sage_quant_k_prep(k, dtype, st, s, nullptr, smooth_k, ws, stream);
 }
 
-int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
-                            const ksana_sage_prep* prep, int smooth_k, void* ws, void* stream) {
+// `part` == nullptr: the chunk sums go to the workspace's own k_part area
+static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
+                        const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -242,6 +273,7 @@ int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const
   hipStream_t hs = static_cast<hipStream_t>(stream);
   const ksana_sage::InTensor kt = in_tensor(k, dtype, st);
   const int bhk = s->B * s->Hkv;
+  if (part == nullptr) part = ws_at<float>(ws, l.k_part);
   ksana_sage::PrepParams pp;
   const ksana_sage::PrepParams* ppp = nullptr;
   if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", st, s->B, s->Lk, ws_at<float>(ws, l.k_rms),
@@ -253,15 +285,38 @@ int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const
     if (e != hipSuccess) return hip_fail(e, "k row statistic launch");
   }
   if (smooth_k) {
-    e = ksana_sage::launch_col_partial(kt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.k_part), l.nch, hs, ppp);
+    e = ksana_sage::launch_col_partial(kt, s->B, s->Hkv, s->Lk, 0, part, l.nch, hs, ppp);
     if (e != hipSuccess) return hip_fail(e, "k column-sum launch");
   }
-  e = ksana_sage::launch_k_mean_finalize(ws_at<float>(ws, l.k_part), bhk, smooth_k ? l.nch : 0, s->Lk, dtype,
+  e = ksana_sage::launch_k_mean_finalize(part, bhk, smooth_k ? l.nch : 0, s->Lk, dtype,
                                          smooth_k, ws_at<float>(ws, l.k_mean), hs);
   if (e != hipSuccess) return hip_fail(e, "k mean finalize launch");
   e = ksana_sage::launch_quant_k(kt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.k_mean),
                                  ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs, ppp);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_k launch");
+}
+
+int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
+                            const ksana_sage_prep* prep, int smooth_k, void* ws, void* stream) {
+  return quant_k_impl(k, dtype, st, s, prep, smooth_k, ws, nullptr, stream);
+}
+
+int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,
+                              void* ws, void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  const int64_t chunk_rows = (int64_t)s->B * s->Hkv * ((s->Lk + ksana_sage::kMeanChunk - 1) / ksana_sage::kMeanChunk);
+  if (chunk_rows > kStaticChunkRows)
+    return fail(KSANA_SAGE_ENOTSUP,
+                "B*Hkv*ceil(Lk/256) = %lld exceeds the %d chunk sums the library's own scratch holds; use "
+                "ksana_sage_quant_k, whose scratch is part of the caller's workspace",
+                (long long)chunk_rows, kStaticChunkRows);
+  // everything else is validated before the device is touched, like in ksana_sage_quant_k
+  if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  float* part = nullptr;
+  if (int rc = static_scratch(&part)) return rc;
+  // every chunk sum the finalisation reads is written by this call's first kernel: nothing to clear
+  return quant_k_impl(k, dtype, st, s, nullptr, smooth_k, ws, part, stream);
 }
 
 int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, void* ws,
