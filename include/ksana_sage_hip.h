@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 8
+#define KSANA_SAGE_ABI_VERSION 9
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -86,6 +86,10 @@ typedef struct ksana_sage_ws_layout {
   uint64_t split_o; /* fp32  [256, 256, D]: scratch of the attention kernel - unnormalised accumulators */
                     /*       of workgroups whose key loop was cut into runs (see ksana_sage_attn_fwd)   */
   uint64_t split_ml;/* fp32  [256, 256, 2]: their running maxima and row sums                           */
+  uint64_t k_sync;  /* int32 [2 * B*Hkv * 32 + 32]: per head a chunk counter and a ready flag (each in a 128-byte */
+                    /*       line of its own) through which the workgroups of the one-read K quantizer meet, then */
+                    /*       one status word                                                                       */
+  uint64_t v_sync;  /* int32, the same for the one-read V quantizer                                                */
   int32_t lq_pad;
   int32_t nqb;
   int32_t nkb;
@@ -135,8 +139,8 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t k_strides[4], con
  * loops, harnesses that forbid it - and therefore cannot grow a workspace for a new shape's scratch.  No counterpart
  * in the reference.  Same arguments, same results bit for bit; the difference is where the kernels' scratch (the
  * per-256-row chunk sums behind the channel means) lives: not in the workspace's k_part area, which this call
- * leaves untouched, but in an 8 MiB array inside the library's own device image.  Limit: B * Hkv * ceil(Lk / 256)
- * <= 16384 (KSANA_SAGE_ENOTSUP beyond).  The call allocates and frees nothing.  All calls on one GPU share that
+ * leaves untouched, but in a 9 MiB array inside the library's own device image.  Limits: B * Hkv * ceil(Lk / 256)
+ * <= 16384 and B * Hkv <= 4096 (KSANA_SAGE_ENOTSUP beyond).  The call allocates and frees nothing.  All calls on one GPU share that
  * array: calls that overlap on one GPU (different streams or threads) race and must be ordered by the caller. */
 int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
                               int smooth_k, void* workspace, void* stream);
@@ -164,6 +168,15 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], con
  * read of V.  smooth_v == 0 is ksana_sage_quant_v. */
 int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[4], const ksana_sage_shape* shape,
                               int smooth_v, void* workspace, void* stream);
+
+/* Did a workgroup of the last ksana_sage_quant_k / ksana_sage_quant_v on this workspace give up waiting for the
+ * others of its head?  Both quantizers read their input once: a workgroup keeps its rows in registers while the
+ * statistic of its head (channel means / column maxima) is gathered from all of them, and that wait is bounded by
+ * a two-second limit so that every kernel ends.  On a GPU shared with nothing else the limit is never met; if it is,
+ * the status word of the stage is 1 and the quantized operands are not to be used.  SYNCHRONISES `stream`, then
+ * copies the two words: a call for tests and diagnostics, not for the hot path.  No counterpart in the reference. */
+int ksana_sage_quant_status(const void* workspace, const ksana_sage_shape* shape, void* stream, int* k_status,
+                            int* v_status);
 
 /* Fused attention on the quantized operands in `workspace`: INT8 QK^T, fp32 online softmax,
  * FP8 PV, output in `dtype` at [B, Lq, Hq, D] with `o_strides`.  Replaces the qattn.* kernel

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -29,6 +29,7 @@ EXPORTS = (
     "ksana_sage_quant_v_smooth",
     "ksana_sage_attn_fwd",
     "ksana_sage_attn_key_split",
+    "ksana_sage_quant_status",
     "ksana_sage_forward",
     "ksana_sage_quant_q_prep",
     "ksana_sage_quant_k_prep",
@@ -48,6 +49,7 @@ class WsLayout(C.Structure):
         for n in (
             "total_bytes", "q_i8", "q_scale", "k_i8", "k_scale", "k_mean",
             "v_fp8", "v_scale", "v_inv", "k_part", "v_part", "q_rms", "k_rms", "v_mean", "split_o", "split_ml",
+            "k_sync", "v_sync",
         )
     ] + [(n, C.c_int32) for n in ("lq_pad", "nqb", "nkb", "nch")]
 
@@ -88,6 +90,7 @@ def _declare(lib):
     lib.ksana_sage_attn_fwd.argtypes, lib.ksana_sage_attn_fwd.restype = [vp, vp, i, st, sp, vp, i, i, vp], i
     ip = C.POINTER(C.c_int)
     lib.ksana_sage_attn_key_split.argtypes, lib.ksana_sage_attn_key_split.restype = [sp, ip, ip], i
+    lib.ksana_sage_quant_status.argtypes, lib.ksana_sage_quant_status.restype = [vp, sp, vp, ip, ip], i
     lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward.restype = i
     pp = C.POINTER(Prep)

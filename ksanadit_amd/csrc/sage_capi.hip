@@ -4,6 +4,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -11,11 +12,15 @@
 #include "sage_kernels.h"
 
 // Scratch of ksana_sage_quant_k_static: the chunk sums of K's channel means, [B * Hkv * ceil(Lk / 256)][128]
-// fp32.  Device memory that belongs to the loaded code object: every GPU the library runs on holds its own copy
-// (8 MiB) at its own address from the first launch on it until the process ends.  In host code the name below is
+// fp32, followed by the counters and flags through which the workgroups of a head meet (cleared by a small kernel
+// at the start of every call).  Device memory that belongs to the loaded code object: every GPU the library runs
+// on holds its own copy (8.1 MiB) at its own address from the first launch on it until the process ends.  In host code the name below is
 // only a handle for hipGetSymbolAddress - the device address it yields is what kernels are given.
 constexpr int kStaticChunkRows = 16384;  // B * Hkv * ceil(Lk / 256) that fit
-static __device__ __align__(256) float scratch[(size_t)kStaticChunkRows * ksana_sage::kD];
+constexpr size_t kStaticPartFloats = (size_t)kStaticChunkRows * ksana_sage::kD;
+constexpr int kStaticHeads = 4096;         // B * Hkv that fit
+constexpr size_t kStaticSyncInts = ksana_sage::sync_words(kStaticHeads);  // per head a counter and a ready flag; a status word
+static __device__ __align__(256) float scratch[kStaticPartFloats + kStaticSyncInts];
 
 namespace {
 
@@ -102,6 +107,25 @@ int static_scratch(float** out) {
   }
   *out = g_scratch_ptr[dev];
   return 0;
+}
+
+// The counter / ready / status words of the K and of the V quantizer inside their areas of sync_words(bhk) ints
+ksana_sage::QuantSync sync_at(int* k_words, int* v_words, int bhk) {
+  const int n = bhk * ksana_sage::kSyncStride;
+  ksana_sage::QuantSync q{};
+  if (k_words) q.k_counter = k_words, q.k_ready = k_words + n, q.k_status = k_words + 2 * n;
+  if (v_words) q.v_counter = v_words, q.v_ready = v_words + n, q.v_status = v_words + 2 * n;
+  return q;
+}
+
+// Which of K and V are quantized by the one-read kernels when the shape allows (otherwise by the two-pass ones):
+// environment variable KSANA_SAGE_ONE_READ = any of the letters "k", "v" ("" = neither); read once.
+bool one_read(char which) {
+  static const char* chosen = [] {
+    const char* e = getenv("KSANA_SAGE_ONE_READ");
+    return e ? e : "v";
+  }();
+  return strchr(chosen, which) != nullptr;
 }
 
 int check_ws(const void* ws) {
@@ -221,6 +245,8 @@ int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout*
   l.v_mean = take(bhk * kD * 4);
   l.split_o = take((uint64_t)kMaxSplitPartials * kAttnQPerWg * kD * 4);
   l.split_ml = take((uint64_t)kMaxSplitPartials * kAttnQPerWg * 2 * 4);
+  l.k_sync = take((uint64_t)sync_words((int)bhk) * 4);
+  l.v_sync = take((uint64_t)sync_words((int)bhk) * 4);
   l.total_bytes = off;
   *out = l;
   return 0;
@@ -262,9 +288,10 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
   return ksana_sage_quant_k_prep(k, dtype, st, s, nullptr, smooth_k, ws, stream);
 }
 
-// `part` == nullptr: the chunk sums go to the workspace's own k_part area
+// `part` == nullptr: the chunk sums and the counters go to the workspace's own k_part / k_sync areas
 static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
-                        const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, void* stream) {
+                        const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, int* sync_words,
+                        void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -274,6 +301,7 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
   const ksana_sage::InTensor kt = in_tensor(k, dtype, st);
   const int bhk = s->B * s->Hkv;
   if (part == nullptr) part = ws_at<float>(ws, l.k_part);
+  if (sync_words == nullptr) sync_words = ws_at<int>(ws, l.k_sync);
   ksana_sage::PrepParams pp;
   const ksana_sage::PrepParams* ppp = nullptr;
   if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", st, s->B, s->Lk, ws_at<float>(ws, l.k_rms),
@@ -284,12 +312,23 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
     e = ksana_sage::launch_row_inv_rms(kt, s->B, s->Hkv, s->Lk, prep->norm_eps, ws_at<float>(ws, l.k_rms), hs);
     if (e != hipSuccess) return hip_fail(e, "k row statistic launch");
   }
+  if (one_read('k')) {
+    // one read of K: chunk sums, the head's mean and the quantization in one kernel, when the shape suits it
+    e = ksana_sage::launch_clear_ints(sync_words, ksana_sage::sync_words(bhk), hs);
+    if (e != hipSuccess) return hip_fail(e, "k counter clear launch");
+    bool used = false;
+    e = ksana_sage::launch_quant_k_fused(kt, s->B, s->Hkv, s->Lk, l.nkb, l.nch, smooth_k ? 1 : 0, part,
+                                         ws_at<float>(ws, l.k_mean), ws_at<int8_t>(ws, l.k_i8),
+                                         ws_at<float>(ws, l.k_scale), sync_at(sync_words, nullptr, bhk), hs, ppp, &used);
+    if (e != hipSuccess) return hip_fail(e, "fused quant_k launch");
+    if (used) return 0;
+  }
   if (smooth_k) {
     e = ksana_sage::launch_col_partial(kt, s->B, s->Hkv, s->Lk, 0, part, l.nch, hs, ppp);
     if (e != hipSuccess) return hip_fail(e, "k column-sum launch");
   }
-  e = ksana_sage::launch_k_mean_finalize(part, bhk, smooth_k ? l.nch : 0, s->Lk, dtype,
-                                         smooth_k, ws_at<float>(ws, l.k_mean), hs);
+  e = ksana_sage::launch_k_mean_finalize(part, bhk, smooth_k ? l.nch : 0, s->Lk, dtype, smooth_k,
+                                         ws_at<float>(ws, l.k_mean), hs, sync_at(sync_words, nullptr, bhk).k_status);
   if (e != hipSuccess) return hip_fail(e, "k mean finalize launch");
   e = ksana_sage::launch_quant_k(kt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.k_mean),
                                  ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs, ppp);
@@ -298,25 +337,27 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
 
 int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                             const ksana_sage_prep* prep, int smooth_k, void* ws, void* stream) {
-  return quant_k_impl(k, dtype, st, s, prep, smooth_k, ws, nullptr, stream);
+  return quant_k_impl(k, dtype, st, s, prep, smooth_k, ws, nullptr, nullptr, stream);
 }
 
 int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,
                               void* ws, void* stream) {
   if (int rc = check_shape(s)) return rc;
   const int64_t chunk_rows = (int64_t)s->B * s->Hkv * ((s->Lk + ksana_sage::kMeanChunk - 1) / ksana_sage::kMeanChunk);
-  if (chunk_rows > kStaticChunkRows)
+  if (chunk_rows > kStaticChunkRows || (int64_t)s->B * s->Hkv > kStaticHeads)
     return fail(KSANA_SAGE_ENOTSUP,
-                "B*Hkv*ceil(Lk/256) = %lld exceeds the %d chunk sums the library's own scratch holds; use "
-                "ksana_sage_quant_k, whose scratch is part of the caller's workspace",
-                (long long)chunk_rows, kStaticChunkRows);
+                "B*Hkv*ceil(Lk/256) = %lld, B*Hkv = %lld: the library's own scratch holds %d chunk sums of %d heads; "
+                "use ksana_sage_quant_k, whose scratch is part of the caller's workspace",
+                (long long)chunk_rows, (long long)s->B * s->Hkv, kStaticChunkRows, kStaticHeads);
   // everything else is validated before the device is touched, like in ksana_sage_quant_k
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
   float* part = nullptr;
   if (int rc = static_scratch(&part)) return rc;
-  // every chunk sum the finalisation reads is written by this call's first kernel: nothing to clear
-  return quant_k_impl(k, dtype, st, s, nullptr, smooth_k, ws, part, stream);
+  // every chunk sum that is read is written earlier in the same call; the counters and flags behind the partial
+  // sums are cleared by the call's first kernel
+  return quant_k_impl(k, dtype, st, s, nullptr, smooth_k, ws, part, reinterpret_cast<int*>(part + kStaticPartFloats),
+                      stream);
 }
 
 int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, void* ws,
@@ -336,6 +377,19 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], con
   const int bhk = s->B * s->Hkv;
   float* v_mean = ws_at<float>(ws, l.v_mean);
   hipError_t e = hipSuccess;
+  if (!smooth_v && one_read('v')) {
+    // one read of V: column maxima, scales and the quantization in one kernel, when the shape suits it
+    int* words = ws_at<int>(ws, l.v_sync);
+    e = ksana_sage::launch_clear_ints(words, ksana_sage::sync_words(bhk), hs);
+    if (e != hipSuccess) return hip_fail(e, "v counter clear launch");
+    bool used = false;
+    e = ksana_sage::launch_quant_v_fused(vt, s->B, s->Hkv, s->Lk, l.nkb, l.nch, ws_at<float>(ws, l.v_part),
+                                         ws_at<float>(ws, l.v_scale),
+                                         ws_at<float>(ws, l.v_inv), v_mean, ws_at<uint8_t>(ws, l.v_fp8),
+                                         sync_at(nullptr, words, bhk), hs, &used);
+    if (e != hipSuccess) return hip_fail(e, "fused quant_v launch");
+    if (used) return 0;
+  }
   if (smooth_v) {
     e = ksana_sage::launch_col_partial(vt, s->B, s->Hkv, s->Lk, 0, ws_at<float>(ws, l.v_part), l.nch, hs);
     if (e != hipSuccess) return hip_fail(e, "v column sum launch");
@@ -349,11 +403,29 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], con
   // without smoothing the mean slot is cleared here: the attention adds whatever it holds
   e = ksana_sage::launch_v_scale_finalize(ws_at<float>(ws, l.v_part), s->B * s->Hkv, l.nch,
                                           ws_at<float>(ws, l.v_scale), ws_at<float>(ws, l.v_inv),
-                                          smooth_v ? nullptr : v_mean, hs);
+                                          smooth_v ? nullptr : v_mean, hs,
+                                          sync_at(nullptr, ws_at<int>(ws, l.v_sync), bhk).v_status);
   if (e != hipSuccess) return hip_fail(e, "v scale finalize launch");
   e = ksana_sage::launch_quant_v(vt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.v_inv),
                                  smooth_v ? v_mean : nullptr, ws_at<uint8_t>(ws, l.v_fp8), hs);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_v launch");
+}
+
+int ksana_sage_quant_status(const void* ws, const ksana_sage_shape* s, void* stream, int* k_status, int* v_status) {
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_ws(ws)) return rc;
+  if (!k_status || !v_status) return fail(KSANA_SAGE_EINVAL, "out-pointer is null");
+  ksana_sage_ws_layout l;
+  ksana_sage_workspace_layout(s, &l);
+  const int bhk = s->B * s->Hkv;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  hipError_t e = hipStreamSynchronize(hs);
+  if (e != hipSuccess) return hip_fail(e, "stream synchronize");
+  const int at = 2 * bhk * ksana_sage::kSyncStride;
+  e = hipMemcpy(k_status, ws_at<int>(ws, l.k_sync) + at, sizeof(int), hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return hip_fail(e, "status copy");
+  e = hipMemcpy(v_status, ws_at<int>(ws, l.v_sync) + at, sizeof(int), hipMemcpyDeviceToHost);
+  return e == hipSuccess ? 0 : hip_fail(e, "status copy");
 }
 
 int ksana_sage_attn_key_split(const ksana_sage_shape* s, int* first_workgroup, int* runs) {

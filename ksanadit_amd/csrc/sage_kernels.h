@@ -51,11 +51,12 @@ hipError_t launch_row_inv_rms(const InTensor& x, int B, int H, int L, float eps,
 // op 0: column sums, 1: column max |x|, 2: column max |x - centre[d]| (centre: [B, H, D])
 hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, float* part, int nch, hipStream_t s,
                               const PrepParams* prep = nullptr, const float* centre = nullptr);
+// status: nullptr, or the quantizer's status word to clear (see QuantSync)
 hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
-                                  hipStream_t s);
+                                  hipStream_t s, int* status = nullptr);
 // zero_mean: nullptr, or the [BH, D] mean slot to clear (V quantized without smoothing)
 hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, float* zero_mean,
-                                   hipStream_t s);
+                                   hipStream_t s, int* status = nullptr);
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
                           float* q_scale, hipStream_t s, const PrepParams* prep = nullptr);
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
@@ -63,6 +64,27 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
 // v_mean: nullptr, or the channel means taken off before scaling (V smoothing)
 hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, const float* v_mean,
                           uint8_t* v_tiles, hipStream_t s);
+
+// Counters and flags of the one-read K / V quantizers, all zero before the launch (launch_clear_ints).  One
+// word per head, kSyncStride words apart so that each sits in a cache line of its own.
+constexpr int kSyncStride = 32;
+constexpr int sync_words(int bh) { return 2 * bh * kSyncStride + kSyncStride; }  // counters, ready flags, status
+struct QuantSync {
+  int* k_counter;  // chunks of the head whose column sums are published
+  int* k_ready;    // non-zero once the head's mean is published
+  int* k_status;   // set to 1 if a workgroup gave up waiting (the results are then not to be trusted)
+  int* v_counter;  // the same three for V: chunks whose column maxima are published,
+  int* v_ready;    // scales published,
+  int* v_status;   // a wait that ran into its limit
+};
+hipError_t launch_clear_ints(int* p, int n, hipStream_t s);
+// One-read quantizers: *used == false means the shape does not suit them and nothing was launched.
+hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb, int nch, int smooth, float* part,
+                                float* k_mean, int8_t* k_tiles, float* k_scale, const QuantSync& sync, hipStream_t s,
+                                const PrepParams* prep, bool* used);
+hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb, int nch, float* part, float* v_scale,
+                                float* v_inv, float* v_mean, uint8_t* v_tiles, const QuantSync& sync, hipStream_t s,
+                                bool* used);
 
 struct AttnParams {
   const int8_t* q_i8;

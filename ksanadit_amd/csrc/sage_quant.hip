@@ -8,6 +8,9 @@
 // specification): plain IEEE fp32 add / sub / mul / div, round-half-even, no contraction.
 #include "sage_kernels.h"
 
+#include <atomic>
+#include <cstdlib>
+
 #include "../../include/ksana_sage_hip.h"
 
 namespace ksana_sage {
@@ -235,29 +238,60 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const uint16_t* base = x + b * sB + h * sH + c16 * 16;
   const RopeLds rl = maybe_stage_rope<PRE>(pp, b, ch * kMeanChunk, kMeanChunk);
-  float rows[kMeanChunk / kSlots][16];
+  float acc[16];
+  if constexpr (PRE) {
+    float rows[kMeanChunk / kSlots][16];
 #pragma unroll
-  for (int i = 0; i < kMeanChunk / kSlots; ++i) {
-    const int row = ch * kMeanChunk + i * kSlots + slot;
-    load_row16<DT>(base + (int64_t)row * sL, row < L, rows[i]);
-    if constexpr (PRE) {
+    for (int i = 0; i < kMeanChunk / kSlots; ++i) {
+      const int row = ch * kMeanChunk + i * kSlots + slot;
+      load_row16<DT>(base + (int64_t)row * sL, row < L, rows[i]);
       if (row < L) prep16<DT>(rows[i], pp, rl, b, row, h, c16);
     }
-    if constexpr (OP == 2) {
-      if (row < L) {
-        const float* cen = centre + ((int64_t)b * H + h) * kD + c16 * 16;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) rows[i][e] = rows[i][e] - cen[e];
+    for (int e = 0; e < 16; ++e) acc[e] = kSum ? rows[0][e] : fabsf(rows[0][e]);
+#pragma unroll
+    for (int i = 1; i < kMeanChunk / kSlots; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[e] = kSum ? acc[e] + rows[i][e] : fmaxf(acc[e], fabsf(rows[i][e]));
+    }
+  } else {
+    // all sixteen loads of the lane are issued first and stay in flight as 16-bit values; they are widened and
+    // folded in row order as they arrive (keeping them as fp32 costs twice the registers and a wave per SIMD)
+    uint4 raw[kMeanChunk / kSlots][2];
+#pragma unroll
+    for (int i = 0; i < kMeanChunk / kSlots; ++i) {
+      const int row = ch * kMeanChunk + i * kSlots + slot;
+      raw[i][0] = raw[i][1] = make_uint4(0, 0, 0, 0);
+      if (row < L) {
+        raw[i][0] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL);
+        raw[i][1] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL + 8);
       }
     }
-  }
-  float acc[16];
+    float cen[16];
+    if constexpr (OP == 2) {
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = kSum ? rows[0][e] : fabsf(rows[0][e]);
+      for (int e = 0; e < 16; ++e) cen[e] = centre[((int64_t)b * H + h) * kD + c16 * 16 + e];
+    }
 #pragma unroll
-  for (int i = 1; i < kMeanChunk / kSlots; ++i) {
+    for (int i = 0; i < kMeanChunk / kSlots; ++i) {
+      const int row = ch * kMeanChunk + i * kSlots + slot;
+      float x[16];
+      widen8<DT>(raw[i][0], x);
+      widen8<DT>(raw[i][1], x + 8);
+      if constexpr (OP == 2) {
+        if (row < L) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = kSum ? acc[e] + rows[i][e] : fmaxf(acc[e], fabsf(rows[i][e]));
+          for (int e = 0; e < 16; ++e) x[e] = x[e] - cen[e];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        if (i == 0)
+          acc[e] = kSum ? x[e] : fabsf(x[e]);
+        else
+          acc[e] = kSum ? acc[e] + x[e] : fmaxf(acc[e], fabsf(x[e]));
+      }
+    }
   }
   // slots of one wave differ in lane bits 3..5
 #pragma unroll
@@ -291,20 +325,38 @@ constexpr int kFinMaxChunks = 96;  // partials staged per pass: 96 x 128 floats 
 
 template <int OP>
 __device__ __forceinline__ float combine_partials(const float* __restrict__ part, int nch, float* s_part) {
-  const int d = threadIdx.x & (kD - 1), sub = threadIdx.x >> 7;  // 8 loader groups
+  const int d = threadIdx.x & (kD - 1);
   float acc = 0.0f;
   bool first = true;
   for (int c0 = 0; c0 < nch; c0 += kFinMaxChunks) {
     const int n = min(kFinMaxChunks, nch - c0);
     __syncthreads();
-    for (int c = sub; c < n; c += kFinThreads / kD) s_part[c * kD + d] = part[(int64_t)(c0 + c) * kD + d];
+    // 96 x 128 floats by 1024 threads: twelve independent loads each, all in flight together
+    float v[kFinMaxChunks * kD / kFinThreads];
+#pragma unroll
+    for (int j = 0; j < kFinMaxChunks * kD / kFinThreads; ++j) {
+      const int idx = (int)threadIdx.x + kFinThreads * j;
+      v[j] = idx < n * kD ? part[(int64_t)c0 * kD + idx] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < kFinMaxChunks * kD / kFinThreads; ++j) s_part[(int)threadIdx.x + kFinThreads * j] = v[j];
     __syncthreads();
     if (threadIdx.x < kD) {
-      for (int c = 0; c < n; ++c) {
-        const float v = s_part[c * kD + d];
-        acc = first ? v : (OP == 0 ? acc + v : fmaxf(acc, v));
+      int c = 0;
+      if (first) {
+        acc = s_part[d];
         first = false;
+        c = 1;
       }
+      // chunk order is part of the specification for the sum; batches of 16 keep the LDS reads ahead of the adds
+      for (; c + 16 <= n; c += 16) {
+        float w[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w[i] = s_part[(c + i) * kD + d];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc = OP == 0 ? acc + w[i] : fmaxf(acc, w[i]);
+      }
+      for (; c < n; ++c) acc = OP == 0 ? acc + s_part[c * kD + d] : fmaxf(acc, s_part[c * kD + d]);
     }
   }
   return acc;
@@ -313,9 +365,10 @@ __device__ __forceinline__ float combine_partials(const float* __restrict__ part
 // chunk sums -> mean rounded to the input dtype, stored widened
 __global__ __launch_bounds__(kFinThreads) void k_mean_finalize_kernel(const float* __restrict__ part, int nch, int L,
                                                                       int dtype, int smooth,
-                                                                      float* __restrict__ k_mean) {
+                                                                      float* __restrict__ k_mean, int* status) {
   __shared__ float s_part[kFinMaxChunks * kD];
   const int bh = blockIdx.x;
+  if (status != nullptr && bh == 0 && threadIdx.x == 0) *status = 0;  // this path has no wait that could expire
   const float tot = combine_partials<0>(part + (int64_t)bh * nch * kD, nch, s_part);
   if (threadIdx.x < kD) {
     const float mean = __fdiv_rn(tot, (float)L);
@@ -327,9 +380,10 @@ __global__ __launch_bounds__(kFinThreads) void k_mean_finalize_kernel(const floa
 __global__ __launch_bounds__(kFinThreads) void v_scale_finalize_kernel(const float* __restrict__ part, int nch,
                                                                        float* __restrict__ v_scale,
                                                                        float* __restrict__ v_inv,
-                                                                       float* __restrict__ zero_mean) {
+                                                                       float* __restrict__ zero_mean, int* status) {
   __shared__ float s_part[kFinMaxChunks * kD];
   const int bh = blockIdx.x;
+  if (status != nullptr && bh == 0 && threadIdx.x == 0) *status = 0;
   const float amax = combine_partials<1>(part + (int64_t)bh * nch * kD, nch, s_part);
   if (threadIdx.x < kD) {
     const bool nz = amax > 0.0f;
@@ -395,18 +449,24 @@ __device__ __forceinline__ float block_max(float v, float* s_red) {
   return fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
 }
 
+// clamp(rne(x * inv), -127, 127) as int8, sixteen at a time.  The product is rounded to fp32 first (the
+// specification's order), clamped (clamping before or after the rounding to an integer gives the same integer), and
+// then rounded to an integer by adding 1.5 * 2^23: at that magnitude the fp32 grid is the integers and the addition
+// rounds to nearest, ties to even, so the low byte of the sum is the two's-complement int8.  Three instructions per
+// value plus three byte-gathers per four, instead of round / clamp / convert / mask / shift / or.
 __device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
   uint32_t w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    uint32_t acc = 0;
+    uint32_t z[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float r = rintf(x[4 * i + j] * inv);
-      r = fminf(fmaxf(r, -127.0f), 127.0f);
-      acc |= ((uint32_t)(int)r & 0xffu) << (8 * j);
+      const float y = __builtin_amdgcn_fmed3f(x[4 * i + j] * inv, -127.0f, 127.0f);
+      z[j] = __float_as_uint(y + 12582912.0f);
     }
-    w[i] = acc;
+    const uint32_t lo = __builtin_amdgcn_perm(z[1], z[0], 0x0c0c0400u);  // bytes 0, 1 <- low bytes of z0, z1
+    const uint32_t hi = __builtin_amdgcn_perm(z[3], z[2], 0x04000c0cu);  // bytes 2, 3 <- low bytes of z2, z3
+    w[i] = lo | hi;
   }
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
@@ -582,6 +642,435 @@ __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __res
   }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// One-read quantizers for K and V.
+//
+// The two-kernel form above reads K (and V) twice: once for the column statistic of the whole
+// sequence, once to quantize.  Here a workgroup keeps its 256-row chunk in registers (as the 16-bit
+// values it loaded: 64 registers per lane) across the point where the statistic of its head becomes
+// known, so every input byte crosses the memory bus once:
+//   1. load the chunk, reduce its columns, publish the chunk's partial result;
+//   2. count the chunk in on its head's counter; the workgroup that finds itself last combines the
+//      partial results (K: in chunk order, which is part of the specification; V: the maximum needs
+//      no order and is taken with an atomic) and raises the head's ready flag;
+//   3. every other workgroup of the head waits for the flag, then all of them quantize from registers.
+// Waiting is safe because workgroups are dispatched in index order: a waiting workgroup only waits for
+// workgroups with indices of the same head, all of which have been dispatched or are next in line on
+// their part of the chip, and the launcher only picks this form when a head's chunks are a fraction
+// of the workgroups the chip holds at once.  The wait is bounded by a wall-clock limit all the same:
+// on expiry the workgroup records it in `status` and carries on with whatever the statistic holds, so
+// every wave ends.
+// ---------------------------------------------------------------------------------------
+constexpr int kChunkRowsPerSlot = kMeanChunk / kSlots;  // 8
+
+// Opaque use+def: what was derived from the 16-bit values before this point (their fp32 forms) is not carried
+// across it; only the 16-bit values themselves stay in registers.
+__device__ __forceinline__ void forget_derived(uint4 (&raw)[kChunkRowsPerSlot][2]) {
+#pragma unroll
+  for (int i = 0; i < kChunkRowsPerSlot; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      asm volatile("" : "+v"(raw[i][j].x), "+v"(raw[i][j].y), "+v"(raw[i][j].z), "+v"(raw[i][j].w));
+}
+
+template <int DT>
+__device__ __forceinline__ uint4 narrow8(const float* x) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (DT == KSANA_SAGE_BF16) {
+      // the values are exactly representable (they went through the half type): truncation is exact
+      w[i] = (__float_as_uint(x[2 * i]) >> 16) | (__float_as_uint(x[2 * i + 1]) & 0xffff0000u);
+    } else {
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      h2 p = {(_Float16)x[2 * i], (_Float16)x[2 * i + 1]};
+      w[i] = __builtin_bit_cast(uint32_t, p);
+    }
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// Communication between workgroups (which may sit behind different L2 caches) goes through accesses that are
+// coherent at device scope by themselves - relaxed device-scope atomics: stores write through, loads are served
+// from the point of coherence - ordered by waiting for their completion (a workgroup-scope fence is that wait
+// plus a compiler barrier).  Device-scope acquire / release fences are avoided on purpose: each one writes back or
+// invalidates a whole L2, and a polling loop built on them starves the loads of every other workgroup.
+__device__ __forceinline__ int load_shared_i32(const int* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared_f32(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void publish_f32(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// every memory access this wave has issued has completed - for the write-through stores and the atomics above:
+// has reached the point of coherence - and the compiler moves no access across
+__device__ __forceinline__ void complete_accesses() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+
+// Thread 0 waits until *flag reaches `want` (or the time limit passes), then the workgroup meets.
+__device__ __forceinline__ void wait_for_head(const int* flag, int want, long long limit_ticks, int* status) {
+  if (threadIdx.x == 0) {
+    if (load_shared_i32(flag) < want) {
+      const long long t0 = wall_clock64();
+      while (load_shared_i32(flag) < want) {
+        __builtin_amdgcn_s_sleep(16);  // ~0.5 us between polls
+        if (wall_clock64() - t0 > limit_ticks) {
+          __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+    complete_accesses();
+  }
+  __syncthreads();
+}
+
+#ifdef KSANA_QUANT_TRACE
+__device__ long long g_quant_trace[16384 * 8];
+#define QTRACE(slot) do { if (threadIdx.x == 0 && blockIdx.x < 16384) g_quant_trace[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define QTRACE(slot) do { } while (0)
+#endif
+
+struct HeadSync {
+  int* counter;      // [B*H][kSyncStride] chunks counted in (one word per head, each in a cache line of its own)
+  int* ready;        // [B*H][kSyncStride] set once the head's statistic is published
+  int* status;       // [1]   set to 1 when a wait ran into its time limit
+  long long limit;   // wall-clock ticks (100 MHz) a workgroup waits at most
+};
+
+// Staging of one head's chunk partials for the workgroup that combines them: kFinStage chunks per
+// pass (16 KiB of LDS), fetched with loads that are all in flight together; the next pass is fetched while this one
+// is combined.
+constexpr int kFinStage = 32;
+constexpr int kFinLoads = kFinStage * kD / kThreads;  // per thread and pass: 32
+
+__device__ __forceinline__ void fetch_partials(const float* hp, int c0, int nch, float (&v)[kFinLoads]) {
+  const int n = (min(kFinStage, nch - c0)) * kD;
+#pragma unroll
+  for (int j = 0; j < kFinLoads; ++j) {
+    const int idx = (int)threadIdx.x + kThreads * j;
+    v[j] = idx < n ? load_shared_f32(hp + (int64_t)c0 * kD + idx) : 0.0f;
+  }
+}
+__device__ __forceinline__ void stage_partials(const float (&v)[kFinLoads], float* s_part) {
+#pragma unroll
+  for (int j = 0; j < kFinLoads; ++j) s_part[(int)threadIdx.x + kThreads * j] = v[j];
+}
+
+template <int DT, bool PRE>
+__global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
+                                                                 int64_t sH, int H, int L, int nkb, int nch,
+                                                                 float* __restrict__ part, float* k_mean, int dtype,
+                                                                 int smooth, int8_t* __restrict__ k_tiles,
+                                                                 float* __restrict__ k_scale, const PrepParams pp,
+                                                                 const HeadSync sy) {
+  const int bh = blockIdx.x / nch, ch = blockIdx.x - bh * nch;
+  const int b = bh / H, h = bh - b * H;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int wave = t >> 6, lane = t & 63;
+  const uint16_t* base = k + b * sB + h * sH + c16 * 16;
+  const RopeLds rl = maybe_stage_rope<PRE>(pp, b, ch * kMeanChunk, kMeanChunk);
+  __shared__ float s_w[4][kD];
+  __shared__ float s_mean[kD];
+  __shared__ float s_red[4][4];
+  __shared__ int s_last;
+  __shared__ float s_part[kFinStage * kD];
+
+  // ---- 1. the chunk, and its column sums in the specified order -------------------------------
+  QTRACE(0);
+  uint4 raw[kChunkRowsPerSlot][2];
+  float acc[16];
+#pragma unroll
+  for (int i = 0; i < kChunkRowsPerSlot; ++i) {
+    const int row = ch * kMeanChunk + i * kSlots + slot;
+    float x[16];
+    if constexpr (PRE) {
+      load_row16<DT>(base + (int64_t)row * sL, row < L, x);
+      if (row < L) prep16<DT>(x, pp, rl, b, row, h, c16);
+      raw[i][0] = narrow8<DT>(x);
+      raw[i][1] = narrow8<DT>(x + 8);
+    } else {
+      raw[i][0] = raw[i][1] = make_uint4(0, 0, 0, 0);
+      if (row < L) {
+        raw[i][0] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL);
+        raw[i][1] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL + 8);
+      }
+      widen8<DT>(raw[i][0], x);
+      widen8<DT>(raw[i][1], x + 8);
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = i == 0 ? x[e] : acc[e] + x[e];
+  }
+  forget_derived(raw);
+#pragma unroll
+  for (int m = 8; m <= 32; m <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = acc[e] + __shfl_xor(acc[e], m);
+  }
+  if (!smooth) {  // uniform: nothing is taken off, nothing to wait for
+    if (t < kD) {
+      s_mean[t] = 0.0f;
+      if (ch == 0) k_mean[bh * kD + t] = 0.0f;
+    }
+    __syncthreads();
+  } else {
+  if (lane < 8) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
+  }
+  __syncthreads();
+  QTRACE(1);
+  if (t < kD) {
+    publish_f32(part + ((int64_t)bh * nch + ch) * kD + t, (s_w[0][t] + s_w[1][t]) + (s_w[2][t] + s_w[3][t]));
+    complete_accesses();  // the partial result is visible chip-wide before this chunk is counted in
+  }
+  __syncthreads();
+  // ---- 2. count the chunk in; the last one of the head publishes the mean -----------------------
+  if (t == 0) {
+    const int before = __hip_atomic_fetch_add(sy.counter + bh * kSyncStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = before == nch - 1;
+    complete_accesses();
+  }
+  QTRACE(2);
+  __syncthreads();
+  if (s_last) {  // uniform
+    const float* hp = part + (int64_t)bh * nch * kD;
+    float tot = 0.0f;
+    float nxt[kFinLoads];
+    fetch_partials(hp, 0, nch, nxt);
+    for (int c0 = 0; c0 < nch; c0 += kFinStage) {
+      const int n = min(kFinStage, nch - c0);
+      __syncthreads();  // the previous pass has been read
+      stage_partials(nxt, s_part);
+      if (c0 + kFinStage < nch) fetch_partials(hp, c0 + kFinStage, nch, nxt);
+      __syncthreads();
+      if (t < kD) {
+        // chunk order is part of the specification
+        if (n == kFinStage) {
+#pragma unroll 16
+          for (int c = 0; c < kFinStage; ++c) tot = (c0 == 0 && c == 0) ? s_part[t] : tot + s_part[c * kD + t];
+        } else {
+          for (int c = 0; c < n; ++c) tot = (c0 == 0 && c == 0) ? s_part[t] : tot + s_part[c * kD + t];
+        }
+      }
+    }
+    if (t < kD) {
+      const float mean = round_to_half_dtype(__fdiv_rn(tot, (float)L), dtype);
+      s_mean[t] = mean;
+      publish_f32(k_mean + bh * kD + t, mean);
+      complete_accesses();
+    }
+    __syncthreads();
+    if (t == 0) __hip_atomic_store(sy.ready + bh * kSyncStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    // ---- 3. everybody else waits for it -----------------------------------------------------------
+    wait_for_head(sy.ready + bh * kSyncStride, 1, sy.limit, sy.status);
+    if (t < kD) s_mean[t] = load_shared_f32(k_mean + bh * kD + t);
+    __syncthreads();
+  }
+  }
+  // ---- 4. quantize the four 64-row tiles of the chunk from registers -----------------------------
+  QTRACE(3);
+#pragma unroll
+  for (int tt = 0; tt < kMeanChunk / kBlkK; ++tt) {
+    const int blk = ch * (kMeanChunk / kBlkK) + tt;
+    if (blk >= nkb) break;  // uniform: the chunk's tail lies beyond the sequence
+    float x[2][16];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = blk * kBlkK + i * kSlots + slot;
+      widen8<DT>(raw[2 * tt + i][0], x[i]);
+      widen8<DT>(raw[2 * tt + i][1], x[i] + 8);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) x[i][e] = row < L ? x[i][e] - s_mean[c16 * 16 + e] : 0.0f;
+      fwht128(x[i], c16);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(x[i][e]));
+    }
+#pragma unroll
+    for (int m = 1; m <= 32; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
+    if (lane == 0) s_red[tt][wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_red[tt][0], s_red[tt][1]), fmaxf(s_red[tt][2], s_red[tt][3]));
+    const bool nz = amax > 0.0f;
+    const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
+    if (t == 0) k_scale[(int64_t)bh * nkb + blk] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
+    int8_t* tile = k_tiles + ((int64_t)bh * nkb + blk) * (int64_t)kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int frag = i * 4 + (c16 >> 1);
+      const int ln = (c16 & 1) * 32 + slot;
+      *reinterpret_cast<uint4*>(tile + (frag * 64 + ln) * 16) = pack_int8x16(x[i], inv);
+    }
+  }
+  QTRACE(4);
+#ifdef KSANA_QUANT_TRACE
+  if (t == 0 && blockIdx.x < 16384) {
+    g_quant_trace[blockIdx.x * 8 + 5] = s_last;
+    g_quant_trace[blockIdx.x * 8 + 6] = bh;
+    g_quant_trace[blockIdx.x * 8 + 7] = ch;
+  }
+#endif
+}
+
+// V: column abs-max of the whole sequence (the last workgroup of a head to arrive takes the maximum over the
+// chunks' maxima - no order to respect - and publishes the scales), then per-channel e4m3 in the transposed tile
+// order of quant_v_kernel.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quant_v_fused_kernel(const uint16_t* __restrict__ v, int64_t sB, int64_t sL,
+                                                                 int64_t sH, int H, int L, int nkb, int nch,
+                                                                 float* __restrict__ part, float* v_scale, float* v_inv,
+                                                                 float* __restrict__ v_mean,
+                                                                 uint8_t* __restrict__ v_tiles, const HeadSync sy) {
+  const int bh = blockIdx.x / nch, ch = blockIdx.x - bh * nch;
+  const int b = bh / H, h = bh - b * H;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int wave = t >> 6, lane = t & 63;
+  const uint16_t* base = v + b * sB + h * sH + c16 * 16;
+  __shared__ float s_w[4][kD];
+  __shared__ float s_inv[kD];
+  __shared__ int s_last;
+  constexpr int kStride = kD + 16;  // LDS row pitch in bytes
+  __shared__ __attribute__((aligned(16))) uint8_t s_v[2][kBlkK * kStride];
+
+  uint4 raw[kChunkRowsPerSlot][2];
+  float acc[16];
+#pragma unroll
+  for (int i = 0; i < kChunkRowsPerSlot; ++i) {
+    const int row = ch * kMeanChunk + i * kSlots + slot;
+    raw[i][0] = raw[i][1] = make_uint4(0, 0, 0, 0);
+    if (row < L) {
+      raw[i][0] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL);
+      raw[i][1] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL + 8);
+    }
+    float x[16];
+    widen8<DT>(raw[i][0], x);
+    widen8<DT>(raw[i][1], x + 8);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = i == 0 ? fabsf(x[e]) : fmaxf(acc[e], fabsf(x[e]));
+  }
+  forget_derived(raw);
+#pragma unroll
+  for (int m = 8; m <= 32; m <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = fmaxf(acc[e], __shfl_xor(acc[e], m));
+  }
+  if (lane < 8) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
+  }
+  __syncthreads();
+  if (t < kD) {
+    publish_f32(part + ((int64_t)bh * nch + ch) * kD + t, fmaxf(fmaxf(s_w[0][t], s_w[1][t]), fmaxf(s_w[2][t], s_w[3][t])));
+    complete_accesses();  // visible chip-wide before this chunk is counted in
+  }
+  __syncthreads();
+  if (t == 0) {
+    const int before = __hip_atomic_fetch_add(sy.counter + bh * kSyncStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = before == nch - 1;
+    complete_accesses();
+  }
+  __syncthreads();
+  if (s_last) {  // uniform
+    // thread t: channel t % 128, chunks of parity t / 128; 32 loads in flight at a time
+    const float* hp = part + (int64_t)bh * nch * kD + (t & (kD - 1));
+    float m = 0.0f;
+    for (int c0 = t >> 7; c0 < nch; c0 += 64) {
+      float v32[32];
+#pragma unroll
+      for (int j = 0; j < 32; ++j) v32[j] = c0 + 2 * j < nch ? load_shared_f32(hp + (int64_t)(c0 + 2 * j) * kD) : 0.0f;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) m = fmaxf(m, v32[j]);
+    }
+    __syncthreads();  // s_w was read above by every thread that needed it
+    s_w[t >> 7][t & (kD - 1)] = m;
+    __syncthreads();
+    if (t < kD) {
+      const float amax = fmaxf(s_w[0][t], s_w[1][t]);
+      const bool nz = amax > 0.0f;
+      const float inv = nz ? __fdiv_rn(448.0f, amax) : 0.0f;
+      s_inv[t] = inv;
+      publish_f32(v_inv + bh * kD + t, inv);
+      v_scale[bh * kD + t] = nz ? __fdiv_rn(amax, 448.0f) : 0.0f;
+      v_mean[bh * kD + t] = 0.0f;
+      complete_accesses();
+    }
+    __syncthreads();
+    if (t == 0) __hip_atomic_store(sy.ready + bh * kSyncStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    wait_for_head(sy.ready + bh * kSyncStride, 1, sy.limit, sy.status);
+    if (t < kD) s_inv[t] = load_shared_f32(v_inv + bh * kD + t);
+    __syncthreads();
+  }
+  float inv[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) inv[e] = s_inv[c16 * 16 + e];
+#pragma unroll
+  for (int tt = 0; tt < kMeanChunk / kBlkK; ++tt) {
+    const int blk = ch * (kMeanChunk / kBlkK) + tt;
+    if (blk >= nkb) break;  // uniform
+    uint8_t* sv = s_v[tt & 1];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = i * kSlots + slot;
+      float x[16];
+      widen8<DT>(raw[2 * tt + i][0], x);
+      widen8<DT>(raw[2 * tt + i][1], x + 8);
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = fminf(fmaxf(x[4 * j + e] * inv[4 * j + e], -448.0f), 448.0f);
+        int packed = 0;
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], packed, false);
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], packed, true);
+        w[j] = (uint32_t)packed;
+      }
+      *reinterpret_cast<uint4*>(&sv[r * kStride + c16 * 16]) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    __syncthreads();  // two staging buffers: the one written two tiles ago was read before the last barrier
+    uint8_t* tile = v_tiles + ((int64_t)bh * nkb + blk) * (int64_t)kTileBytes;
+#pragma unroll
+    for (int i = 0; i < kTileBytes / 16 / kThreads; ++i) {
+      const int oc = i * kThreads + t;
+      const int dt = oc >> 7, th = (oc >> 6) & 1, ln = oc & 63;
+      const int hh = ln >> 5, d = dt * 32 + (ln & 31);
+      uint32_t w[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint32_t a = 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int row = 32 * th + 8 * g + 4 * hh + c;
+          a |= (uint32_t)sv[row * kStride + d] << (8 * c);
+        }
+        w[g] = a;
+      }
+      *reinterpret_cast<uint4*>(tile + oc * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+}
+
+#ifdef KSANA_QUANT_TRACE
+}  // namespace
+}  // namespace ksana_sage
+extern "C" int ksana_debug_quant_trace(long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(ksana_sage::g_quant_trace), (size_t)n * sizeof(long long));
+}
+namespace ksana_sage {
+namespace {
+#endif
+
+__global__ void clear_ints_kernel(int* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
 }  // namespace
 
 #define KSANA_DISPATCH_DT(dtype, ...)            \
@@ -641,14 +1130,14 @@ hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, fl
 }
 
 hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int dtype, int smooth, float* k_mean,
-                                  hipStream_t s) {
-  k_mean_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, L, dtype, smooth, k_mean);
+                                  hipStream_t s, int* status) {
+  k_mean_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, L, dtype, smooth, k_mean, status);
   return hipGetLastError();
 }
 
 hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, float* zero_mean,
-                                   hipStream_t s) {
-  v_scale_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, v_scale, v_inv, zero_mean);
+                                   hipStream_t s, int* status) {
+  v_scale_finalize_kernel<<<dim3(BH), dim3(kFinThreads), 0, s>>>(part, nch, v_scale, v_inv, zero_mean, status);
   return hipGetLastError();
 }
 
@@ -686,6 +1175,88 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
     }
   });
   return hipGetLastError();
+}
+
+namespace {
+// Workgroups of `kernel` (256 threads, `lds` bytes of dynamic LDS) the current device holds at once.
+// (0 when the runtime cannot tell: the caller then takes the two-pass kernels.)  The answer for a launch
+// without dynamic LDS is kept per device and kernel.
+template <typename K>
+int resident_workgroups(K kernel, size_t lds) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int per_cu = 0, dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  if (lds == 0) {
+    const int c = cached[dev].load(std::memory_order_acquire);
+    if (c > 0) return c;
+  }
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (lds == 0) cached[dev].store(per_cu * cus, std::memory_order_release);
+  return per_cu * cus;
+}
+constexpr long long kWaitLimitTicks = 200000000;  // 2 s of the 100 MHz wall clock
+
+}  // namespace
+
+hipError_t launch_clear_ints(int* p, int n, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  clear_ints_kernel<<<dim3((n + 255) / 256), dim3(256), 0, s>>>(p, n);
+  return hipGetLastError();
+}
+
+// The one-read forms are used when a head's chunks are at most half of what the chip holds at once (see the
+// comment above the kernels); *used tells the caller whether anything was launched.
+hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb, int nch, int smooth, float* part,
+                                float* k_mean, int8_t* k_tiles, float* k_scale, const QuantSync& sync, hipStream_t s,
+                                const PrepParams* prep, bool* used) {
+  *used = false;
+  if ((int64_t)B * H * nch > INT32_MAX) return hipSuccess;
+  const dim3 grid(B * H * nch), block(kThreads);
+  const HeadSync sy{sync.k_counter, sync.k_ready, sync.k_status, kWaitLimitTicks};
+  const PrepParams none{};
+  hipError_t e = hipSuccess;
+  KSANA_DISPATCH_DT(k.dtype, {
+    if (prep == nullptr) {
+      const int resident = resident_workgroups(quant_k_fused_kernel<DT, false>, 0);
+      if (2 * nch <= resident) {
+        quant_k_fused_kernel<DT, false><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
+                                                                k.dtype, smooth, k_tiles, k_scale, none, sy);
+        *used = true;
+      }
+    } else {
+      PrepParams pp = *prep;
+      const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
+      if (2 * nch <= resident_workgroups(quant_k_fused_kernel<DT, true>, lds)) {
+        quant_k_fused_kernel<DT, true><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
+                                                                 k.dtype, smooth, k_tiles, k_scale, pp, sy);
+        *used = true;
+      }
+    }
+  });
+  if (*used) e = hipGetLastError();
+  return e;
+}
+
+hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb, int nch, float* part, float* v_scale,
+                                float* v_inv, float* v_mean, uint8_t* v_tiles, const QuantSync& sync, hipStream_t s,
+                                bool* used) {
+  *used = false;
+  if ((int64_t)B * H * nch > INT32_MAX) return hipSuccess;
+  const dim3 grid(B * H * nch), block(kThreads);
+  const HeadSync sy{sync.v_counter, sync.v_ready, sync.v_status, kWaitLimitTicks};
+  hipError_t e = hipSuccess;
+  KSANA_DISPATCH_DT(v.dtype, {
+    const int resident = resident_workgroups(quant_v_fused_kernel<DT>, 0);
+    if (2 * nch <= resident) {
+      quant_v_fused_kernel<DT><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, nch, part, v_scale, v_inv,
+                                                       v_mean, v_tiles, sy);
+      *used = true;
+    }
+  });
+  if (*used) e = hipGetLastError();
+  return e;
 }
 
 hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, const float* v_mean,

@@ -256,6 +256,16 @@ def quant_v(v: torch.Tensor, ws: SageWorkspace, smooth_v: bool = False) -> None:
     _capi.check(rc, "ksana_sage_quant_v")
 
 
+def quant_status(ws: SageWorkspace) -> tuple[int, int]:
+    """``(k_status, v_status)`` of the last K / V quantization on ``ws``: 0, or 1 when a workgroup gave up waiting for
+    the others of its head (see ``ksana_sage_quant_status``).  Synchronises the current stream; for tests."""
+    ks, vs = C.c_int(-1), C.c_int(-1)
+    rc = _capi.load().ksana_sage_quant_status(ws.ptr, C.byref(ws.shape), _stream_ptr(ws.blob.device), C.byref(ks),
+                                              C.byref(vs))
+    _capi.check(rc, "ksana_sage_quant_status")
+    return ks.value, vs.value
+
+
 def _k_lens_arg(k_lens, batch: int, device: torch.device):
     """``k_lens`` as the int32 device array the library reads (kept alive by the caller's reference)."""
     if k_lens is None:

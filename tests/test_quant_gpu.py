@@ -20,6 +20,7 @@ def _run_quant(q, k, v, dev, sm_scale=None, smooth_k=True):
     sage_ops.quant_k(kd, ws, smooth_k)
     sage_ops.quant_v(vd, ws)
     torch.cuda.synchronize()
+    assert sage_ops.quant_status(ws) == (0, 0), "a quantizer workgroup gave up waiting for its head"
     return ws
 
 
@@ -110,6 +111,40 @@ def test_quantizer_bit_exact_workloads(hip_device, name, heads, seq):
     print(f"workload {name} heads={heads}", flush=True)
     q, k, v = make_inputs(name, heads=heads, seq=seq)
     _check_against_oracle(q, k, v, hip_device)
+
+
+def test_quantizer_bit_exact_past_the_one_read_limit(hip_device):
+    """K and V are quantized by kernels that read them once as long as the 256-row chunks of one head are at most
+    half of the workgroups the chip holds at a time (1024 on an MI355X); beyond that - here 547 chunks per head - the
+    two-pass kernels take over.  Same bits either way; Q (no statistic over the sequence) is kept short."""
+    Lk = 140000
+    print(f"case long Lk={Lk}", flush=True)
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn((1, 100, 1, 128), generator=g).to(torch.bfloat16)
+    k = (torch.randn((1, Lk, 1, 128), generator=g) + 2.0 * torch.randn((1, 1, 1, 128), generator=g)).to(torch.bfloat16)
+    v = (torch.randn((1, Lk, 1, 128), generator=g) * 1.5).to(torch.bfloat16)
+    _check_against_oracle(q, k, v, hip_device)
+
+
+def test_quantizers_repeat_bit_for_bit(hip_device):
+    """The one-read kernels meet through counters in the workspace: a second run on the same workspace (the
+    counters are cleared by each call) and a run on a fresh one give the same bytes."""
+    q, k, v = make_inputs("qwen_cfg", heads=3)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    blobs = []
+    for rep in range(3):
+        if rep == 2:
+            ws = sage_ops.workspace_for(qd, kd)
+            ws.blob.fill_(0xFF)  # counters that start from garbage would never reach their target
+        sage_ops.quant_k(kd, ws)
+        sage_ops.quant_v(vd, ws)
+        torch.cuda.synchronize()
+        assert sage_ops.quant_status(ws) == (0, 0)
+        blobs.append([ws.k_tiles.clone(), ws.k_scale.clone(), ws.k_mean.clone(), ws.v_tiles.clone(), ws.v_scale.clone()])
+    for other in blobs[1:]:
+        for a, b_ in zip(blobs[0], other):
+            assert torch.equal(a, b_)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
