@@ -23,8 +23,10 @@ METRIC = "Sage-attn effective TFLOPS & % INT8/FP8 MFMA peak, Wan-14B 480p (L=327
 MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense INT8 (POP/s) = dense FP8 (PFLOP/s) = 5.0e15 /s
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from
-# two rocprofv3 --pmc runs, factors from a 1 GiB device copy in the same runs (profiles/sage_attn_fwd_kernel_wan14b_480p.md)
+# two rocprofv3 --pmc runs, factors from a 1 GiB device copy in the same runs.  A constant from that profile, not a
+# counter read in this run (counters need rocprofv3 around the process).
 ATTN_TRAFFIC_BYTES = {"wan14b_480p": 1808505 * 1024}
+ATTN_TRAFFIC_SOURCE = "profiles/sage_attn_fwd_kernel_wan14b_480p.md (rocprofv3 --pmc, not this run)"
 
 
 def parse():
@@ -38,6 +40,7 @@ def parse():
     ap.add_argument("--skip-extra", action="store_true", help="leave out the block-sparse and norm+RoPE legs (they run after the timed steps)")
     ap.add_argument("--skip-block-sparse", action="store_true", help="leave out the block-sparse leg only")
     ap.add_argument("--skip-causal", action="store_true", help="leave out the causal leg only (it launches the same kernel instantiation as the block-sparse leg)")
+    ap.add_argument("--skip-other-workloads", action="store_true", help="leave out the attention timings at the other measured shapes")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
     return ap.parse_args()
 
@@ -81,6 +84,154 @@ def cpu_baseline(workload, target_s: float):
     }
 
 
+def pctl(xs, q):
+    xs = sorted(xs)
+    return xs[min(len(xs) - 1, max(0, int(round(q * (len(xs) - 1)))))]
+
+
+def spread(xs, digits=4):
+    """median, 10th and 90th percentile of a list of per-step times"""
+    return {"median": round(pctl(xs, 0.5), digits), "p10": round(pctl(xs, 0.1), digits), "p90": round(pctl(xs, 0.9), digits)}
+
+
+def device_inputs(w, dev, Lq=None, Lk=None):
+    """q, k, v of a workload's distributions drawn on the device (seeded): for legs whose timing, not whose values,
+    is reported - drawing 3 x 387 M values on the host would take longer than everything else together."""
+    g = torch.Generator(device=dev).manual_seed(w.seed)
+    Lq = w.L if Lq is None else Lq
+    Lk = w.L if Lk is None else Lk
+
+    def draw(L, offset, outliers):
+        x = torch.randn((w.B, L, w.H, w.D), generator=g, device=dev, dtype=torch.float32)
+        if w.text_tokens:
+            x[:, : min(w.text_tokens, L)] *= w.text_std
+        if offset:
+            x += torch.randn((w.H, w.D), generator=g, device=dev) * w.k_offset_std
+        if outliers and w.outlier_p > 0:
+            m = torch.rand(x.shape, generator=g, device=dev) < w.outlier_p
+            x = torch.where(m, x * w.outlier_gain, x)
+        return x.to(torch.bfloat16)
+
+    return draw(Lq, False, True), draw(Lk, True, True), draw(Lk, False, False)
+
+
+def time_attention(sage_ops, ws, out, iters, **kw):
+    """median / p10 / p90 of the attention call on the operands in ``ws`` (HIP events on the launch stream)"""
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
+    sage_ops.attn_fwd(ws, out, **kw)
+    torch.cuda.synchronize()
+    for e in ev:
+        e[0].record()
+        sage_ops.attn_fwd(ws, out, **kw)
+        e[1].record()
+    torch.cuda.synchronize()
+    return [e[0].elapsed_time(e[1]) for e in ev]
+
+
+def mfma_probe(dev, iters=5):
+    """What the matrix pipe sustains on the attention kernel's own MFMA mix with nothing else running."""
+    import ctypes as C
+
+    from ksanadit_amd import _capi
+
+    lib = _capi.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    scratch = torch.empty(cus * 512, dtype=torch.float32, device=dev)
+    ops = C.c_double(0.0)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    times = []
+    for i in range(iters + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _capi.check(lib.ksana_sage_mfma_probe(scratch.data_ptr(), scratch.numel() * 4, cus, 20000, stream, C.byref(ops)),
+                    "ksana_sage_mfma_probe")
+        e1.record()
+        torch.cuda.synchronize()
+        if i:
+            times.append(e0.elapsed_time(e1))
+    return round(ops.value / (pctl(times, 0.5) * 1e-3) / 1e12, 1)
+
+
+def op_end_to_end(w, q, k, v, iters=7):
+    """One call through KsanaAttentionOp as a model block makes it: backend adaptor, workspace from torch's allocator,
+    three quantizers, attention, output tensor."""
+    from ksanadit_amd import KsanaAttentionBackend, KsanaAttentionConfig, pick_attn_op
+
+    op = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN))(num_heads=w.H, head_size=w.D)
+    op(q, k, v)
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        o = op(q, k, v)
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1))
+        del o
+    return spread(times)
+
+
+def other_workloads(sage_ops, dev, pwl, iters=7):
+    """Attention-kernel time at the other measured shapes (parity-test shapes; values drawn on the device)."""
+    from ksanadit_amd.workloads import WORKLOADS, Workload
+
+    cases = [(WORKLOADS[n], None, None) for n in ("wan5b_720p", "wan14b_720p", "qwen_cfg")]
+    # WanCrossAttention: every video token attends to the 512 text tokens (wan_model.py:233-251, text_len 512)
+    cases.append((Workload("wan14b_480p_cross_attn", 1006, 1, 40, 32760), 32760, 512))
+    res = {}
+    for w, Lq, Lk in cases:
+        q, k, v = device_inputs(w, dev, Lq, Lk)
+        ws = sage_ops.workspace_for(q, k)
+        out = torch.empty_like(q)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        sm = w.D**-0.5
+        sage_ops.quant_q(q, ws, sm), sage_ops.quant_k(k, ws, True), sage_ops.quant_v(v, ws)
+        torch.cuda.synchronize()
+        ev[0].record()
+        sage_ops.quant_q(q, ws, sm), sage_ops.quant_k(k, ws, True), sage_ops.quant_v(v, ws)
+        ev[1].record()
+        times = time_attention(sage_ops, ws, out, iters, pwl_exp2=pwl)
+        flops = 4.0 * w.B * w.H * q.shape[1] * k.shape[1] * w.D
+        ms = pctl(times, 0.5)
+        res[w.name] = {"shape": f"B={w.B} H={w.H} Lq={q.shape[1]} Lk={k.shape[1]} D={w.D}", "attn_kernel_ms": spread(times),
+                       "attn_kernel_tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                       "frac_of_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                       "quantizer_ms": round(ev[0].elapsed_time(ev[1]), 4)}
+        del q, k, v, ws, out
+        torch.cuda.empty_cache()
+    return res
+
+
+def radial_leg(sage_ops, dev, pwl, iters=5):
+    """The block-sparse call with the mask the radial backend builds (backends/radial_mask.py, which reproduces the
+    reference's generator bit for bit) on a latent grid that backend accepts: height and width multiples of 16
+    (radial_sage_attn.py:123-124), here 21 frames of 64 x 112 -> 32 x 56 tokens, L = 37632, H = 40."""
+    from ksanadit_amd.backends.radial_mask import kernel_block_mask, radial_block_mask
+    from ksanadit_amd.config import KsanaRadialSageAttentionConfig
+    from ksanadit_amd.workloads import Workload
+
+    cfg = KsanaRadialSageAttentionConfig()
+    frames, tpf = 21, 32 * 56
+    w = Workload("wan14b_radial_grid", 1007, 1, 40, frames * tpf, outlier_p=1e-3)
+    q, k, v = device_inputs(w, dev)
+    ws = sage_ops.workspace_for(q, k)
+    out = torch.empty_like(q)
+    sm = w.D**-0.5
+    sage_ops.quant_q(q, ws, sm), sage_ops.quant_k(k, ws, True), sage_ops.quant_v(v, ws)
+    pattern = radial_block_mask(w.L, w.L, frames, cfg.block_size, cfg.decay_factor)
+    mask = kernel_block_mask(pattern, cfg.block_size, w.L).to(dev)
+    density = float(mask.float().mean())
+    dense = pctl(time_attention(sage_ops, ws, out, iters, pwl_exp2=pwl), 0.5)
+    times = time_attention(sage_ops, ws, out, iters, pwl_exp2=pwl, block_mask=mask)
+    ms = pctl(times, 0.5)
+    return {"mask": f"radial_block_mask(L={w.L}, frames={frames}, block_size={cfg.block_size}, decay_factor={cfg.decay_factor})",
+            "shape": f"B=1 H=40 L={w.L} D=128", "density": round(density, 4), "attn_kernel_ms": spread(times),
+            "dense_attn_kernel_ms": round(dense, 4),
+            "tflops_on_kept_blocks": round(w.flops * density / (ms * 1e-3) / 1e12, 2),
+            "kept_block_rate_vs_dense": round((w.flops * density / ms) / (w.flops / dense), 3)}
+
+
 # (frames, height, width) of the latent token grid behind each Wan workload's sequence length
 WAN_GRIDS = {"cpu_plumbing": (3, 20, 26), "wan5b_720p": (31, 22, 40), "wan14b_480p": (21, 30, 52),
              "wan14b_720p": (21, 45, 80)}
@@ -111,35 +262,22 @@ def block_sparse_leg(sage_ops, w, ws, out, grid, pwl, iters):
     density = float(mask.float().mean())
     pairs = mask[: mask.shape[0] // 2 * 2].view(-1, 2, mask.shape[1]).amax(dim=1)  # what a 256-row workgroup walks
     density_wg = float(pairs.float().mean())
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
-    sage_ops.attn_fwd(ws, out, pwl_exp2=pwl, block_mask=mask)
-    torch.cuda.synchronize()
-    for e in ev:
-        e[0].record()
-        sage_ops.attn_fwd(ws, out, pwl_exp2=pwl, block_mask=mask)
-        e[1].record()
-    torch.cuda.synchronize()
-    ms = sum(e[0].elapsed_time(e[1]) for e in ev) / iters
+    times = time_attention(sage_ops, ws, out, iters, pwl_exp2=pwl, block_mask=mask)
+    ms = pctl(times, 0.5)
     return {
         "mask": "radial-style, 128x64 blocks, broadcast over heads",
         "density": round(density, 4),
         "density_per_256_row_workgroup": round(density_wg, 4),
         "attn_kernel_ms": round(ms, 4),
+        "attn_kernel_ms_spread": spread(times),
         "tflops_on_kept_blocks": round(w.flops * density / (ms * 1e-3) / 1e12, 2),
     }
 
 
 def causal_leg(sage_ops, w, ws, out, pwl, iters):
     """Outside the timed step: the same kernel with causal masking (half of the score matrix)."""
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
-    sage_ops.attn_fwd(ws, out, causal=True, pwl_exp2=pwl)
-    torch.cuda.synchronize()
-    for e in ev:
-        e[0].record()
-        sage_ops.attn_fwd(ws, out, causal=True, pwl_exp2=pwl)
-        e[1].record()
-    torch.cuda.synchronize()
-    ms = sum(e[0].elapsed_time(e[1]) for e in ev) / iters
+    times = time_attention(sage_ops, ws, out, iters, causal=True, pwl_exp2=pwl)
+    ms = pctl(times, 0.5)
     kept = (w.L + 1) / (2.0 * w.L)  # fraction of (query, key) pairs on or below the diagonal
     return {"attn_kernel_ms": round(ms, 4), "tflops_on_kept_pairs": round(w.flops * kept / (ms * 1e-3) / 1e12, 2)}
 
@@ -268,8 +406,11 @@ def main() -> int:
     t1 = time.perf_counter()
 
     ms_step = (t1 - t0) * 1e3 / args.steps
-    quant_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    attn_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    quant_times = [e[0].elapsed_time(e[1]) for e in events]
+    attn_times = [e[1].elapsed_time(e[2]) for e in events]
+    step_times = [e[0].elapsed_time(e[2]) for e in events]
+    quant_ms = sum(quant_times) / args.steps
+    attn_ms = sum(attn_times) / args.steps
     attn_tflops = w.flops / (attn_ms * 1e-3) / 1e12
     n = w.elements
     quant_bytes = 9.0 * n  # q, k, v read once as 16-bit, written once as 8-bit
@@ -294,6 +435,10 @@ def main() -> int:
         "attn_kernel_tflops": round(attn_tflops, 2),
         "pct_mfma_peak": round(100.0 * attn_tflops / MFMA_PEAK_TFLOPS, 2),
         "quantizer_ms": round(quant_ms, 4),
+        # per-step times between HIP events on the launch stream: the means above, and how the steps scatter
+        "step_ms_spread": spread(step_times),
+        "attn_kernel_ms_spread": spread(attn_times),
+        "quantizer_ms_spread": spread(quant_times),
         "roofline": {
             "kernel": "sage_attn_fwd_kernel",
             "bound": "mfma",
@@ -302,9 +447,10 @@ def main() -> int:
             "unit": "TFLOP/s",
             "frac": round(attn_tflops / MFMA_PEAK_TFLOPS, 4),
             "traffic": ATTN_TRAFFIC_BYTES.get(w.name),
+            "traffic_source": ATTN_TRAFFIC_SOURCE if w.name in ATTN_TRAFFIC_BYTES else None,
         },
         "quantizer_roofline": {
-            "kernels": "col_partial x2, finalize x2, quant_q, quant_k, quant_v",
+            "kernels": "quant_q; col_partial + k_mean_finalize + quant_k; quant_v_fused (one read of V)",
             "bound": "hbm",
             "achieved": round(quant_gbs, 1),
             "peak": HBM_PEAK_GBS,
@@ -316,6 +462,12 @@ def main() -> int:
     grid = WAN_GRIDS.get(w.name)
     if args.skip_extra:
         grid = None
+    else:
+        # the matrix pipe alone, same process, same clocks
+        rec["mfma_microbench_tflops"] = mfma_probe(dev)
+        rec["roofline"]["frac_of_mfma_microbench"] = round(attn_tflops / rec["mfma_microbench_tflops"], 4)
+        # what a model block pays per call: the op, its adaptor, workspace allocation, quantizers, attention
+        rec["op_e2e_ms"] = op_end_to_end(w, q, k, v)
     if grid is not None and w.L <= 131072:
         if not args.skip_block_sparse:
             rec["block_sparse"] = block_sparse_leg(sage_ops, w, ws, out, grid, args.pwl_exp2, max(3, args.steps // 2))
@@ -323,6 +475,12 @@ def main() -> int:
             rec["causal"] = causal_leg(sage_ops, w, ws, out, args.pwl_exp2, max(3, args.steps // 2))
     if grid is not None and w.B == 1:
         rec["prep_quantizer"] = prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, max(3, args.steps // 2))
+    if not args.skip_extra and not args.skip_other_workloads:
+        del q, k, v, ws, out
+        torch.cuda.empty_cache()
+        if not args.skip_block_sparse:
+            rec["block_sparse_radial"] = radial_leg(sage_ops, dev, args.pwl_exp2)
+        rec["other_workloads"] = other_workloads(sage_ops, dev, args.pwl_exp2)
     if args.cpu_seconds > 0:
         rec["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
     print(json.dumps(rec))

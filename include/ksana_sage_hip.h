@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 9
+#define KSANA_SAGE_ABI_VERSION 10
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -215,6 +215,14 @@ int ksana_sage_attn_fwd_masked(void* workspace, void* o, int dtype, const int64_
  * *runs runs; *runs == 0 means no cut.  For tools that want to mirror the kernel's rounding exactly (the test
  * emulation does); no counterpart in the reference. */
 int ksana_sage_attn_key_split(const ksana_sage_shape* shape, int* first_workgroup, int* runs);
+
+/* Measurement aid, no counterpart in the reference: launches `workgroups` workgroups of 8 waves that each issue, `steps`
+ * times, the attention kernel's matrix instructions per key tile (8 INT8 + 5 FP8 MFMAs) on register operands and
+ * nothing else.  `scratch` receives workgroups * 512 floats (so the work is not optimised away); *ops_per_launch is the
+ * number of operations (multiply-add = 2) one launch performs.  Time it with events on `stream`: the rate is what the
+ * matrix pipe sustains at the clock it holds under this load. */
+int ksana_sage_mfma_probe(void* scratch, uint64_t scratch_bytes, int workgroups, int steps, void* stream,
+                          double* ops_per_launch);
 
 /* The whole path in one call: quant_q, quant_k, quant_v, attn_fwd on `stream`.
  * Replaces sageattn(q, k, v, tensor_layout="NHD", is_causal=causal) (sage_attn.py:75-81). */

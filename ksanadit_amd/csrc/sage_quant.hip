@@ -9,7 +9,6 @@
 #include "sage_kernels.h"
 
 #include <atomic>
-#include <cstdlib>
 
 #include "../../include/ksana_sage_hip.h"
 
@@ -727,13 +726,6 @@ __device__ __forceinline__ void wait_for_head(const int* flag, int want, long lo
   __syncthreads();
 }
 
-#ifdef KSANA_QUANT_TRACE
-__device__ long long g_quant_trace[16384 * 8];
-#define QTRACE(slot) do { if (threadIdx.x == 0 && blockIdx.x < 16384) g_quant_trace[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
-#else
-#define QTRACE(slot) do { } while (0)
-#endif
-
 struct HeadSync {
   int* counter;      // [B*H][kSyncStride] chunks counted in (one word per head, each in a cache line of its own)
   int* ready;        // [B*H][kSyncStride] set once the head's statistic is published
@@ -780,7 +772,6 @@ __global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t*
   __shared__ float s_part[kFinStage * kD];
 
   // ---- 1. the chunk, and its column sums in the specified order -------------------------------
-  QTRACE(0);
   uint4 raw[kChunkRowsPerSlot][2];
   float acc[16];
 #pragma unroll
@@ -822,7 +813,6 @@ __global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t*
     for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
   }
   __syncthreads();
-  QTRACE(1);
   if (t < kD) {
     publish_f32(part + ((int64_t)bh * nch + ch) * kD + t, (s_w[0][t] + s_w[1][t]) + (s_w[2][t] + s_w[3][t]));
     complete_accesses();  // the partial result is visible chip-wide before this chunk is counted in
@@ -834,7 +824,6 @@ __global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t*
     s_last = before == nch - 1;
     complete_accesses();
   }
-  QTRACE(2);
   __syncthreads();
   if (s_last) {  // uniform
     const float* hp = part + (int64_t)bh * nch * kD;
@@ -873,7 +862,6 @@ __global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t*
   }
   }
   // ---- 4. quantize the four 64-row tiles of the chunk from registers -----------------------------
-  QTRACE(3);
 #pragma unroll
   for (int tt = 0; tt < kMeanChunk / kBlkK; ++tt) {
     const int blk = ch * (kMeanChunk / kBlkK) + tt;
@@ -907,14 +895,6 @@ __global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t*
       *reinterpret_cast<uint4*>(tile + (frag * 64 + ln) * 16) = pack_int8x16(x[i], inv);
     }
   }
-  QTRACE(4);
-#ifdef KSANA_QUANT_TRACE
-  if (t == 0 && blockIdx.x < 16384) {
-    g_quant_trace[blockIdx.x * 8 + 5] = s_last;
-    g_quant_trace[blockIdx.x * 8 + 6] = bh;
-    g_quant_trace[blockIdx.x * 8 + 7] = ch;
-  }
-#endif
 }
 
 // V: column abs-max of the whole sequence (the last workgroup of a head to arrive takes the maximum over the
@@ -1055,16 +1035,6 @@ __global__ __launch_bounds__(kThreads) void quant_v_fused_kernel(const uint16_t*
     }
   }
 }
-
-#ifdef KSANA_QUANT_TRACE
-}  // namespace
-}  // namespace ksana_sage
-extern "C" int ksana_debug_quant_trace(long long* host, int n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(ksana_sage::g_quant_trace), (size_t)n * sizeof(long long));
-}
-namespace ksana_sage {
-namespace {
-#endif
 
 __global__ void clear_ints_kernel(int* p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
