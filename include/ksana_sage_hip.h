@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 10
+#define KSANA_SAGE_ABI_VERSION 11
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -39,7 +39,7 @@ extern "C" {
 /* error codes */
 #define KSANA_SAGE_OK 0
 #define KSANA_SAGE_EINVAL (-1)   /* bad shape, stride, alignment, dtype or null pointer      */
-#define KSANA_SAGE_ENOTSUP (-2)  /* valid request this build does not implement (D != 128, causal with Lq != Lk) */
+#define KSANA_SAGE_ENOTSUP (-2)  /* valid request this build does not implement (D != 128, sizes beyond its limits) */
 #define KSANA_SAGE_EHIP (-3)     /* the HIP runtime reported an error at launch               */
 
 /* flags of the attention entry points */
@@ -187,8 +187,8 @@ int ksana_sage_quant_status(const void* workspace, const ksana_sage_shape* shape
  * repeated calls give identical bits.  The quantized operands in the workspace are only read; the runs' scratch
  * (split_o, split_ml) is the one part of it this call writes.
  * causal: non-zero lets query row i attend to keys [0, i] only (the is_causal of sage_attn.py:75-81 and of
- * sdpa.py:62-79), on top of k_lens and the block mask.  Defined for Lq == Lk (KSANA_SAGE_ENOTSUP otherwise:
- * for other shapes the libraries anchor the triangle at different corners) and Lk <= 131072.
+ * sdpa.py:62-79), on top of k_lens and the block mask; for Lq != Lk the triangle is anchored at the top left corner,
+ * as torch's scaled_dot_product_attention anchors it (sdpa.py:62-79 is the accuracy anchor of this path).  Lk <= 131072.
  * k_lens: NULL, or a device array of B int32: batch b attends to keys [0, k_lens[b]) only
  * (clamped to [0, Lk]; a batch without keys gets zeros).  Same meaning as the k_lens the
  * reference's callers pass (wan_model.py:182-189) and its variable-length backend honours
@@ -209,6 +209,16 @@ int ksana_sage_attn_fwd_masked(void* workspace, void* o, int dtype, const int64_
                                const ksana_sage_shape* shape, const int8_t* block_mask,
                                const int64_t mask_strides[2], const int32_t* k_lens, int causal, int flags,
                                void* stream);
+
+/* ksana_sage_attn_fwd_masked with a per-batch count of query rows as well: q_lens is NULL or a device array of B int32;
+ * rows [0, q_lens[b]) of batch b (clamped to [0, Lq]) are computed, the rows from there to Lq are written as zeros and
+ * cost nothing.  The q_lens of the reference's backends (flash_attn.py:120-124 packs the first q_lens[b] rows of every
+ * batch entry before its variable-length call; sdpa.py:52-57 accepts and ignores the argument, like the Sage adaptor,
+ * which NULL reproduces).  Everything else as in ksana_sage_attn_fwd_masked. */
+int ksana_sage_attn_fwd_varlen(void* workspace, void* o, int dtype, const int64_t o_strides[4],
+                               const ksana_sage_shape* shape, const int8_t* block_mask,
+                               const int64_t mask_strides[2], const int32_t* q_lens, const int32_t* k_lens,
+                               int causal, int flags, void* stream);
 
 /* How ksana_sage_attn_fwd cuts `shape` on the current device (dense, non-causal calls): the 256-row query blocks
  * numbered *first_workgroup and up - numbering (b * Hq + h) * ceil(Lq/256) + block - have their key loop cut into

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -36,6 +36,7 @@ EXPORTS = (
     "ksana_sage_quant_k_prep",
     "ksana_sage_forward_prep",
     "ksana_sage_attn_fwd_masked",
+    "ksana_sage_attn_fwd_varlen",
     "ksana_sage_forward_masked",
 )
 
@@ -104,6 +105,8 @@ def _declare(lib):
     ms = C.POINTER(C.c_int64)
     lib.ksana_sage_attn_fwd_masked.argtypes = [vp, vp, i, st, sp, vp, ms, vp, i, i, vp]
     lib.ksana_sage_attn_fwd_masked.restype = i
+    lib.ksana_sage_attn_fwd_varlen.argtypes = [vp, vp, i, st, sp, vp, ms, vp, vp, i, i, vp]
+    lib.ksana_sage_attn_fwd_varlen.restype = i
     lib.ksana_sage_forward_masked.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, ms, vp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward_masked.restype = i
 

@@ -12,7 +12,9 @@ Differences, all deliberate:
   ``D ** -0.5``; the two agree for every caller because attention_op.py:39 defaults to that value);
 * ``k_lens``: ignored by default, exactly like the reference's adaptor (sage_attn.py:58-84).  Constructed with
   ``honor_k_lens=True`` the backend limits batch ``b`` to its first ``k_lens[b]`` keys, which is what the reference's
-  variable-length backend does with the same argument (flash_attn.py:131-139) and what padded batches need;
+  variable-length backend does with the same argument (flash_attn.py:131-139) and what padded batches need; the same
+  switch makes it honour ``q_lens`` (flash_attn.py:120-124): rows of batch ``b`` from ``q_lens[b]`` on are not computed
+  and come out as zeros;
 * ``out_dtype`` (constructor argument, opt-in): the result is written in that half dtype instead of the query's, which
   folds the cast the Wan block applies before its output projection (wan_model.py:197-204) into the kernel;
 * ``smooth_v`` (constructor argument, opt-in): V is quantized around its channel means, which the kernel adds back to
@@ -81,9 +83,10 @@ class SageAttentionImpl(KsanaAttentionBackendImpl):
         if original_dtype not in (torch.float16, torch.bfloat16):
             query, key, value = (t.to(torch.bfloat16) for t in (query, key, value))
         k_lens = kwargs.get("k_lens") if self.honor_k_lens else None
+        q_lens = kwargs.get("q_lens") if self.honor_k_lens else None
         output = sageattn(query, key, value, tensor_layout="NHD", is_causal=self.causal, sm_scale=self.softmax_scale,
                           k_lens=k_lens, out_dtype=self.out_dtype, pwl_exp2=self.pwl_exp2,
-                          smooth_v=self.smooth_v)
+                          smooth_v=self.smooth_v, q_lens=q_lens)
         if self.out_dtype is not None:
             return output
         return output if output.dtype == original_dtype else output.to(original_dtype)

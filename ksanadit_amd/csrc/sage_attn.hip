@@ -135,7 +135,11 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction: keep it scalar
   const int l32 = lane & 31, hh = lane >> 5;
   const int q0 = qwg * kAttnQPerWg + wave * 32;
-  const bool active = q0 < p.Lq;  // wave-uniform; inactive waves only help move tiles
+  // query rows [0, lq) of this batch take part: all of them, or the caller's per-batch count; the rows from lq up
+  // to Lq exist in the output and are written as zeros
+  int lq = p.Lq;
+  if (p.q_lens != nullptr) lq = min(max(p.q_lens[b], 0), p.Lq);  // uniform: a scalar load
+  const bool active = q0 < lq;  // wave-uniform; inactive waves only help move tiles
 
   // keys [0, lk) of this batch take part: all of them, or the caller's per-batch count
   int lk = p.Lk;
@@ -154,7 +158,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const int per = (tiles + p.n_split - 1) / p.n_split;
     tile0 = split * per;
     const int tile1 = min(tiles, tile0 + per);
-    if (tile0 >= tile1) {  // nothing in this run (few tiles, or a batch entry without keys): an empty partial
+    if (tile0 >= tile1 || qwg * kAttnQPerWg >= lq) {  // nothing in this run (few tiles, a batch entry without keys, or no query row): an empty partial
       if (active) {
         const int row = wave * 32 + l32;
         float* po = p.split_o + ((int64_t)blockIdx.x * kAttnQPerWg + row) * kD + 64 * hh;
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     }
     lk = min(lk, tile1 * kBlkK) - tile0 * kBlkK;  // from here on the run is the whole key sequence
   } else {
-    if (lk == 0) {
+    if (lk == 0 || qwg * kAttnQPerWg >= lq) {  // no key, or none of the workgroup's rows takes part
       write_zero_rows();
       return;
     }
@@ -357,6 +361,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
       tile_barrier();
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (!kSplit) write_zero_rows();  // rows in [lq, Lq), if any (the merge kernel writes them for cut blocks)
     return;
   }
 
@@ -605,9 +610,9 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     return;
   }
   // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
-  // a mask row that allows none of its keys has an empty sum: its rows are zeros, not 0/0
-  const float inv_l = (!kSparse || lacc[0] > 0.0f) ? 1.0f / lacc[0] : 0.0f;
   const int q = q0 + l32;
+  // zero for a mask row that allows none of its keys (an empty sum, not 0/0) and for rows at or beyond lq
+  const float inv_l = ((!kSparse || lacc[0] > 0.0f) && q < lq) ? 1.0f / lacc[0] : 0.0f;
   if (q < p.Lq) {
     uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
     const float* vs = p.v_scale + (int64_t)bhk * kD;
@@ -643,6 +648,11 @@ __global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p
   const int row = blockIdx.y * 8 + (threadIdx.x >> 5), d = (threadIdx.x & 31) * 4;
   const int q = qwg * kAttnQPerWg + row;
   if (q >= p.Lq) return;
+  uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
+  if (p.q_lens != nullptr && q >= min(max(p.q_lens[b], 0), p.Lq)) {  // a row that does not take part: zeros
+    *reinterpret_cast<uint2*>(orow + d) = make_uint2(0, 0);
+    return;
+  }
   const float2* ml = reinterpret_cast<const float2*>(p.split_ml) + (int64_t)item * p.n_split * kAttnQPerWg + row;
   const float* po = p.split_o + ((int64_t)item * p.n_split * kAttnQPerWg + row) * kD + d;
   float m = -INFINITY;
@@ -661,7 +671,6 @@ __global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p
   const float keep_mean = l > 0.0f ? 1.0f : 0.0f;
   const float4 s4 = *reinterpret_cast<const float4*>(p.v_scale + (int64_t)bhk * kD + d);
   const float4 m4 = *reinterpret_cast<const float4*>(p.v_mean + (int64_t)bhk * kD + d);
-  uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
   store4<DT>(orow + d, acc.x * inv_l * s4.x + m4.x * keep_mean, acc.y * inv_l * s4.y + m4.y * keep_mean,
              acc.z * inv_l * s4.z + m4.z * keep_mean, acc.w * inv_l * s4.w + m4.w * keep_mean);
 }

@@ -144,12 +144,10 @@ int check_mask(const ksana_sage_shape* s, const int8_t* block_mask, const int64_
   return 0;
 }
 
-// Causal masking is defined for self-attention shapes only: with Lq != Lk the libraries disagree on which
-// corner the triangle is anchored to, and no caller of this path needs it.
+// Causal masking: query row i sees keys [0, i] (the triangle is anchored at the top left corner, as torch's SDPA
+// anchors it when Lq != Lk); the kernel keeps its list of key tiles in LDS, which bounds Lk.
 int check_causal(const ksana_sage_shape* s, int causal) {
   if (!causal) return 0;
-  if (s->Lq != s->Lk)
-    return fail(KSANA_SAGE_ENOTSUP, "causal masking needs Lq == Lk (got %d and %d)", s->Lq, s->Lk);
   if (s->Lk > ksana_sage::kSparseMaxKeyTiles * ksana_sage::kBlkK)
     return fail(KSANA_SAGE_ENOTSUP, "Lk=%d exceeds %d with causal masking (the tile list is kept in LDS)", s->Lk,
                 ksana_sage::kSparseMaxKeyTiles * ksana_sage::kBlkK);
@@ -445,6 +443,12 @@ int ksana_sage_attn_fwd(void* ws, void* o, int dtype, const int64_t o_st[4], con
 int ksana_sage_attn_fwd_masked(void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
                                const int8_t* block_mask, const int64_t mask_st[2], const int32_t* k_lens, int causal,
                                int flags, void* stream) {
+  return ksana_sage_attn_fwd_varlen(ws, o, dtype, o_st, s, block_mask, mask_st, nullptr, k_lens, causal, flags, stream);
+}
+
+int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
+                               const int8_t* block_mask, const int64_t mask_st[2], const int32_t* q_lens,
+                               const int32_t* k_lens, int causal, int flags, void* stream) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_mask(s, block_mask, mask_st)) return rc;
   if (int rc = check_causal(s, causal)) return rc;
@@ -452,6 +456,7 @@ int ksana_sage_attn_fwd_masked(void* ws, void* o, int dtype, const int64_t o_st[
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
   if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
+  if (reinterpret_cast<uintptr_t>(q_lens) & 3) return fail(KSANA_SAGE_EINVAL, "q_lens is not 4-byte aligned");
   ksana_sage_ws_layout l;
   ksana_sage_workspace_layout(s, &l);
   ksana_sage::AttnParams p;
@@ -470,6 +475,7 @@ int ksana_sage_attn_fwd_masked(void* ws, void* o, int dtype, const int64_t o_st[
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;
   p.exact_exp2 = (flags & KSANA_SAGE_FLAG_PWL_EXP2) ? 0 : 1;
   p.k_lens = k_lens;
+  p.q_lens = q_lens;
   p.block_mask = block_mask;
   p.mask_sB = block_mask ? mask_st[0] : 0;
   p.mask_sH = block_mask ? mask_st[1] : 0;

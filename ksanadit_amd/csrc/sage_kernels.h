@@ -98,11 +98,12 @@ struct AttnParams {
   int B, Hq, Hkv, Lq, Lk, lq_pad, nkb;
   int exact_exp2;  // 1: exp2 on the transcendental unit; 0: piecewise-linear e4m3 code (faster)
   const int32_t* k_lens;  // optional [B]: batch b attends to keys [0, clamp(k_lens[b], 0, Lk)); nullptr = all
+  const int32_t* q_lens;  // optional [B]: query rows [0, clamp(q_lens[b], 0, Lq)) of batch b are computed, the rest zeros
   // optional block mask, int8 [B, Hq, ceil(Lq/128), ceil(Lk/64)] (rows contiguous): non-zero = the 128 query
   // rows attend to the 64 keys; nullptr = dense
   const int8_t* block_mask;
   int64_t mask_sB, mask_sH;  // element strides of the two leading dims (0 broadcasts)
-  int causal;  // 1: query row i attends to keys [0, i] only (on top of k_lens and the block mask)
+  int causal;  // 1: query row i attends to keys [0, i] only (on top of k_lens and the block mask), whatever Lq and Lk
   // scratch for workgroups cut into runs of key tiles (nullptr: never cut): per partial 256 rows x 128 fp32
   // accumulators, and per row its running maximum and row sum; room for kMaxSplitPartials partials
   float* split_o;

@@ -266,13 +266,13 @@ def quant_status(ws: SageWorkspace) -> tuple[int, int]:
     return ks.value, vs.value
 
 
-def _k_lens_arg(k_lens, batch: int, device: torch.device):
-    """``k_lens`` as the int32 device array the library reads (kept alive by the caller's reference)."""
+def _k_lens_arg(k_lens, batch: int, device: torch.device, name: str = "k_lens"):
+    """``k_lens`` / ``q_lens`` as the int32 device array the library reads (kept alive by the caller's reference)."""
     if k_lens is None:
         return None
     k_lens = torch.as_tensor(k_lens)
     if k_lens.dim() != 1 or k_lens.numel() != batch:
-        raise ValueError(f"k_lens must hold one length per batch entry ({batch}), got shape {tuple(k_lens.shape)}")
+        raise ValueError(f"{name} must hold one length per batch entry ({batch}), got shape {tuple(k_lens.shape)}")
     return k_lens.to(device=device, dtype=torch.int32).contiguous()
 
 
@@ -307,13 +307,14 @@ def key_split_plan(ws: SageWorkspace):
 
 
 def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False,
-             k_lens=None, block_mask=None) -> torch.Tensor:
+             k_lens=None, block_mask=None, q_lens=None) -> torch.Tensor:
     """Attention on the quantized operands in ``ws``.  ``k_lens`` (optional, one int per batch entry): batch ``b``
     attends to keys ``[0, k_lens[b])`` only, the meaning the reference's callers give it (wan_model.py:182-189,
     flash_attn.py:131-139); a batch entry without keys yields zeros.  ``block_mask`` (optional, int8/bool
     ``[B, H, ceil(Lq/128), ceil(Lk/64)]``, leading dims may broadcast): block ``(i, j)`` non-zero lets query rows
     ``128 i ..`` attend to keys ``64 j ..`` - the ``mask_id`` of the reference's block-sparse call
-    (radial_sage_attn.py:170-176)."""
+    (radial_sage_attn.py:170-176).  ``q_lens`` (optional, one int per batch entry): only the first ``q_lens[b]`` query
+    rows of batch ``b`` are computed, the rest of the output is zeros (flash_attn.py:120-124 packs exactly those rows)."""
     _require_hip(out)
     if out.dim() != 4:
         raise ValueError("out must be [B, Lq, H, D]")
@@ -321,10 +322,12 @@ def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp
     lib = _capi.load()
     flags = _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0
     kl = _k_lens_arg(k_lens, out.shape[0], out.device)
+    ql = _k_lens_arg(q_lens, out.shape[0], out.device, "q_lens")
     s = ws.shape
     mask, mask_st = _block_mask_arg(block_mask, s.B, s.Hq, s.Lq, s.Lk, out.device)
-    rc = lib.ksana_sage_attn_fwd_masked(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
+    rc = lib.ksana_sage_attn_fwd_varlen(ws.ptr, out.data_ptr(), _DTYPES[out.dtype], _strides(out), C.byref(ws.shape),
                                         None if mask is None else mask.data_ptr(), mask_st,
+                                        None if ql is None else ql.data_ptr(),
                                         None if kl is None else kl.data_ptr(), int(causal), flags,
                                         _stream_ptr(out.device))
     _capi.check(rc, "ksana_sage_attn_fwd")
@@ -346,10 +349,13 @@ def sageattn(
     block_mask=None,
     out_dtype: torch.dtype | None = None,
     smooth_v: bool = False,
+    q_lens=None,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
 
     ``k_lens`` (optional, one int per batch entry) limits batch ``b`` to its first ``k_lens[b]`` keys.
+    ``q_lens`` (optional, likewise): only the first ``q_lens[b]`` query rows of batch ``b`` are computed; the others
+    come out as zeros.
     ``prep`` (optional, "NHD" only): q and k are the raw projections and the block's RMSNorm + RoPE are applied
     while they are read (see ``WanPrep``).
     ``block_mask`` (optional): block-sparse attention, see ``attn_fwd`` (not together with ``prep``).
@@ -385,7 +391,12 @@ def sageattn(
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)
     flags = (_capi.FLAG_PWL_EXP2 if pwl_exp2 else 0) | (_capi.FLAG_SMOOTH_V if smooth_v else 0)
-    if out_dtype is not None and out_dtype != q.dtype:
+    if q_lens is not None and (out_dtype is None or out_dtype == q.dtype):
+        out_dtype_eff = q.dtype
+    else:
+        out_dtype_eff = out_dtype
+    if out_dtype_eff is not None and (out_dtype_eff != q.dtype or q_lens is not None):
+        out_dtype = out_dtype_eff
         if out_dtype not in _DTYPES:
             raise ValueError(f"out_dtype must be float16 or bfloat16, got {out_dtype}")
         # the quantized operands carry no dtype: quantize from q's, write the result in the other
@@ -393,7 +404,7 @@ def sageattn(
         quant_k(k, ws, smooth_k, prep=prep)
         quant_v(v, ws, smooth_v)
         out = torch.empty((B, Lq, Hq, D), dtype=out_dtype, device=q.device)
-        attn_fwd(ws, out, causal=is_causal, pwl_exp2=pwl_exp2, k_lens=kl, block_mask=block_mask)
+        attn_fwd(ws, out, causal=is_causal, pwl_exp2=pwl_exp2, k_lens=kl, block_mask=block_mask, q_lens=q_lens)
         return out.transpose(1, 2) if tensor_layout == "HND" else out
     if block_mask is not None:
         if prep is not None:

@@ -57,8 +57,9 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     the 256-row query blocks numbered ``first_workgroup`` and up (numbering: ``(b * H + h) * ceil(Lq/256) + block``)
     into ``runs`` equal runs of key tiles, walks each run on its own and merges the partial results; probabilities are
     then rounded relative to the run's own running maximum, which this mirrors.
-    ``causal`` (``Lq == Lk`` only): row ``i`` sees keys ``[0, i]``; in the online form a row sits out the tiles that
-    start after it and sees a prefix of the tile that holds its own position.
+    ``causal``: row ``i`` sees keys ``[0, i]`` (for ``Lq != Lk`` too: the triangle sits in the top left corner, as
+    torch's ``is_causal`` puts it); in the online form a row sits out the tiles that start after it and sees a prefix
+    of the tile that holds its own position.
     """
     B, H, Lq, D = q_i8.shape
     Hkv, Lk = k_i8.shape[1], k_i8.shape[2]
@@ -84,8 +85,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
             s_int = q_i8[b, h].float() @ k_i8[b, hk].float().t()
             s = s_int * (qs_row[b, h][:, None] * ks_col[b, hk][None, :])
             if causal:
-                if Lq != Lk:
-                    raise NotImplementedError("causal masking with Lq != Lk")
+                # key <= row, the triangle anchored at the top left corner whatever Lq and Lk (torch's is_causal)
                 mask = torch.ones(Lq, Lk, dtype=torch.bool).tril()
                 s = s.masked_fill(~mask, float("-inf"))
             vf = v_fp8[b, hk].float()
@@ -117,7 +117,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                         act = bm[b, h, :, j0 // BLKK].repeat_interleave(128)[:Lq][:, None]
                     allow = None  # keys of this tile each row may see
                     if causal:
-                        # key <= row (Lq == Lk); a row before the tile's first key sits the step out, the rows
+                        # key <= row; a row before the tile's first key sits the step out, the rows
                         # on the diagonal see a prefix of the tile
                         allow = torch.arange(j0, j1)[None, :] <= rows
                         act = allow[:, :1] if act is None else (act & allow[:, :1])

@@ -286,9 +286,59 @@ def test_causal_with_k_lens_block_mask_backend_and_limits(hip_device):
     sage = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN))(num_heads=H, head_size=128, causal=True)
     sdpa = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.TORCH_SDPA))(num_heads=H, head_size=128, causal=True)
     assert _cos(sage(qd, kd, vd).cpu(), sdpa(qd, kd, vd).cpu()) >= COS_MIN
-    # other shapes: the libraries disagree on the corner the triangle hangs from, so the call is refused
-    with pytest.raises(NotImplementedError):
-        sage_ops.sageattn(qd[:, :100], kd, vd, is_causal=True)
+
+
+@pytest.mark.parametrize("Lq,Lk", [(100, 400), (400, 100), (513, 130), (64, 1000), (300, 299)])
+def test_causal_with_different_query_and_key_lengths(hip_device, Lq, Lk):
+    """Row i sees keys [0, i]: the triangle sits in the top left corner, as torch's SDPA (the accuracy anchor,
+    sdpa.py:62-79) puts it when the two lengths differ.  Rows past the last key see every key."""
+    print(f"case causal Lq={Lq} Lk={Lk}", flush=True)
+    q, k, v = _rand_qkv(2, Lq, Lk, 2, 2, seed=900 + Lq)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    out = sage_ops.sageattn(qd, kd, vd, workspace=ws, is_causal=True).cpu()
+    assert torch.isfinite(out.float()).all()
+    emul = _emul_from_ws(ws, Lq, Lk, q.dtype, causal=True)
+    scale = max(emul.float().abs().max().item(), 1e-3)
+    assert (out.float() - emul.float()).abs().max() <= 2e-2 * scale
+    assert _cos(out, emul) > 0.99999
+    assert _cos(out, sdpa_ref(q, k, v, causal=True)) >= COS_MIN
+    if Lq > Lk:  # the rows below the triangle are plain attention over all keys
+        dense = sage_ops.attn_fwd(ws, torch.empty_like(qd)).cpu()
+        first_full = -(-Lk // 64) * 64  # the first row whose wave sees every key tile whole
+        if first_full < Lq:
+            assert _cos(out[:, first_full:], dense[:, first_full:]) > 0.99999
+
+
+@pytest.mark.parametrize("shape,q_lens", [((2, 300, 200, 2), [100, 0]), ((2, 513, 513, 3), [513, 257]),
+                                          ((3, 256, 640, 1), [1, 255, 256]), ((1, 1560, 1560, 6), [700])])
+def test_q_lens_limits_the_rows_that_are_computed(hip_device, shape, q_lens):
+    """q_lens as flash_attn.py:120-124 reads it: only the first q_lens[b] query rows of batch b take part.  Those
+    rows come out bit for bit as without the argument, the others as zeros - with and without a block mask, with causal
+    masking, and on a shape whose last query blocks are cut into key runs (the fourth)."""
+    B, Lq, Lk, H = shape
+    print(f"case q_lens B={B} Lq={Lq} Lk={Lk} H={H} q_lens={q_lens}", flush=True)
+    q, k, v = _rand_qkv(B, Lq, Lk, H, H, seed=500 + Lq)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    full = sage_ops.sageattn(qd, kd, vd, workspace=ws).cpu()
+    nq, nk = -(-Lq // 128), -(-Lk // 64)
+    mask = (torch.rand((nq, nk), generator=torch.Generator().manual_seed(Lq)) < 0.7).to(torch.int8)
+    mask[:, 0] = 1
+    variants = [dict(), dict(block_mask=mask)] + ([dict(causal=True)] if Lq == Lk else [])
+    for kw in variants:
+        want = sage_ops.attn_fwd(ws, torch.empty_like(qd), **kw).cpu() if kw else full
+        got = torch.full_like(qd, float("nan"))
+        sage_ops.attn_fwd(ws, got, q_lens=q_lens, **kw)
+        got = got.cpu()
+        for b, n in enumerate(q_lens):
+            assert torch.equal(got[b, :n], want[b, :n]), f"batch {b} rows below q_lens differ ({kw.keys()})"
+            assert (got[b, n:] == 0).all(), f"batch {b} rows from q_lens on are not zero ({kw.keys()})"
+    via_op = sage_ops.sageattn(qd, kd, vd, q_lens=q_lens).cpu()
+    for b, n in enumerate(q_lens):
+        assert torch.equal(via_op[b, :n], full[b, :n]) and (via_op[b, n:] == 0).all()
+    with pytest.raises(ValueError):
+        sage_ops.attn_fwd(ws, torch.empty_like(qd), q_lens=[1] * (B + 1))
 
 
 def test_radial_backend_gates_and_masks(hip_device):
@@ -518,15 +568,40 @@ def test_workloads_vs_cpu_sdpa_oracle(hip_device, name, heads, exact):
     out = sage_ops.sageattn(*(t.to(hip_device) for t in (q, k, v)), pwl_exp2=not exact).cpu()
     c = _cos(out, ref)
     err = (out.float() - ref.float()).abs()
-    print(f"{name}: cos={c:.6f} max_abs={err.max().item():.4e} mean_abs={err.mean().item():.4e} ref_max={ref.float().abs().max().item():.3f}", flush=True)
+    ref_max = ref.float().abs().max().item()
+    p999 = err.flatten().kthvalue(max(1, int(0.999 * err.numel()))).values.item()
+    print(f"{name}: cos={c:.6f} max_abs={err.max().item():.4e} ({err.max().item() / ref_max:.4f} of max|O|) "
+          f"p99.9={p999:.4e} ({p999 / ref_max:.4f}) mean_abs={err.mean().item():.4e} ({err.mean().item() / ref_max:.5f}) "
+          f"ref_max={ref_max:.3f}", flush=True)
     assert c >= COS_MIN
     if name == "cpu_plumbing":
         assert err.max().item() <= (MAX_ABS_FLAT if exact else 2 * MAX_ABS_FLAT)
     else:
-        # peaked attention (outlier / text tokens): |O| ~ |V| ~ 1-5, so a max-abs bound has to be
-        # relative: two e4m3 roundings (2 x 2^-4) plus int8 logit noise on near-tied top keys
-        assert err.max().item() <= 0.3 * ref.float().abs().max().item()
-        assert err.mean().item() <= 0.04 * ref.float().abs().mean().item() + 1e-3
+        max_rel, p999_rel, mean_rel = SCHEME_BUDGET[name][0 if exact else 1]
+        assert err.max().item() <= max_rel * ref_max
+        assert p999 <= p999_rel * ref_max
+        assert err.mean().item() <= mean_rel * ref_max
+
+
+# Stated tolerance against SDPA on the peaked workloads, as fractions of max|O_sdpa|: (worst element, 99.9th
+# percentile, mean) for the exact-exp2 and the piecewise-linear path.  Where the numbers come from: the CPU
+# decomposition oracle/error_budget.py on the same seeded inputs (``python -m oracle.error_budget <workload> <heads>``)
+# gives, for the scheme itself (int8 Q/K + e4m3 P + e4m3 V, bf16 result):
+#     wan14b_480p, 1 head : worst 0.179 (0.184 with the int8 step alone), p99.9 0.0330, mean 0.00402
+#     qwen_cfg,    6 heads: worst 0.093 (0.083 with the int8 step alone), p99.9 0.0225, mean 0.00185
+# The worst elements are int8 logit noise, not fp8 rounding: a query row with a x20 outlier meets keys that carry
+# outliers too; their Hadamard-spread outlier components cancel in the exact product, their rounding errors do not
+# (logit error up to 0.6 nats), and two such keys share the row's weight almost evenly.  A K scale per 32 keys leaves
+# that element where it is (same module, k_block = 32).  The gates are the scheme's figures plus 10 % (worst element;
+# the kernel's online softmax rounds P relative to the running maximum, the decomposition relative to the final one)
+# and plus 30 % (percentile, mean); the piecewise-linear path gets what it measured plus the same margins.
+SCHEME_BUDGET = {
+    "wan14b_480p": ((0.20, 0.043, 0.0052), (0.22, 0.045, 0.0056)),
+    "qwen_cfg": ((0.105, 0.029, 0.0024), (0.12, 0.033, 0.0029)),
+}
+# Full shapes, all heads, per group of 8 heads against torch SDPA on the GPU: worst element over 8 x L x 128 outputs
+# relative to that group's max|O| (the tail of the same int8 effect over 8 - 40 times more rows than above)
+FULL_SIZE_WORST = {"wan14b_480p": 0.20, "wan14b_720p": 0.22, "qwen_cfg": 0.15}
 
 
 @pytest.mark.parametrize("name", ["wan5b_720p", "wan14b_480p", "wan14b_720p", "qwen_cfg"])
@@ -553,6 +628,8 @@ def test_full_size_properties(hip_device, name):
     assert c_min >= COS_MIN
     if name == "wan5b_720p":
         assert (out.float() - sdpa(q, k, v).float()).abs().max().item() <= MAX_ABS_FLAT
+    else:
+        assert worst <= FULL_SIZE_WORST[name]
     # rows of P sum to one: V == 1 -> O == 1 (e4m3 holds 1.0 exactly; the normaliser is fp32)
     ones = torch.ones_like(v)
     o1 = sage_ops.sageattn(q, k, ones)

@@ -113,9 +113,12 @@ def test_entry_points_validate_before_touching_the_gpu():
     odd = _capi.Strides(64 * 2 * 128, 2 * 128 + 4, 128, 1)
     assert lib.ksana_sage_quant_q(fake, _capi.BF16, odd, C.byref(shape), 0.1, fake, null) == _capi.EINVAL
     assert lib.ksana_sage_quant_q(fake, _capi.BF16, st, C.byref(shape), 0.1, null, null) == _capi.EINVAL  # workspace
-    rect = _capi.Shape(1, 2, 2, 64, 128, 128)  # causal masking is defined for Lq == Lk only
-    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(rect), null, 1, 0, null) == _capi.ENOTSUP
-    assert b"Lq == Lk" in lib.ksana_sage_last_error()
+    long_k = _capi.Shape(1, 2, 2, 64, 131073, 128)  # causal masking keeps its tile list in LDS: Lk <= 131072
+    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(long_k), null, 1, 0, null) == _capi.ENOTSUP
+    assert b"causal" in lib.ksana_sage_last_error()
+    assert lib.ksana_sage_attn_fwd_varlen(fake, fake, _capi.BF16, st, C.byref(shape), null, None, C.c_void_p(0x1002), null,
+                                          0, 0, null) == _capi.EINVAL  # q_lens alignment
+    assert b"q_lens" in lib.ksana_sage_last_error()
     assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), null, 0, 0x10, null) == _capi.EINVAL  # flags
     assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), C.c_void_p(0x1002), 0, 0, null) == _capi.EINVAL  # k_lens alignment
     assert lib.ksana_sage_forward(fake, fake, null, fake, _capi.BF16, st, st, st, st, C.byref(shape), null, 0.1, 1, 0, 0, fake, null) == _capi.EINVAL
