@@ -51,6 +51,11 @@ extern "C" {
 #define KSANA_SAGE_FLAG_SMOOTH_V 2 /* ksana_sage_forward* only: quantize V with its channel means taken off   */
                                    /* (see ksana_sage_quant_v_smooth).                                        */
 
+#define KSANA_SAGE_FLAG_WG_4_WAVES 4 /* attention entry points: force workgroups of 4 waves (128 query rows, two per   */
+#define KSANA_SAGE_FLAG_WG_8_WAVES 8 /* compute unit) / of 8 waves (256 rows, one per unit) instead of the library's   */
+                                     /* own choice (4 with a block mask, causal masking or Lk <= 1024).  Same results  */
+                                     /* up to the rounding of the key-run merge; for measurements.                     */
+
 /* rows per int8 scale: Q per token, K per 64 keys (sage_sla.py:190,204 uses (128, 64) off-Hopper;
  * the per-token Q scale is free in this kernel's operand layout and tighter) */
 #define KSANA_SAGE_BLKQ 1

@@ -17,6 +17,8 @@ BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
 FLAG_PWL_EXP2 = 1
 FLAG_SMOOTH_V = 2
+FLAG_WG_4_WAVES = 4
+FLAG_WG_8_WAVES = 8
 
 EXPORTS = (
     "ksana_sage_abi_version",

@@ -34,15 +34,28 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kWaves = 8;
-constexpr int kThreadsAttn = kWaves * 64;
+// Two shapes of workgroup: 8 waves = 256 query rows with an 8-stage tile ring (one workgroup holds a compute unit:
+// every K/V tile copied serves 256 rows), and 4 waves = 128 query rows with a 4-stage ring, two of which share a
+// compute unit - they run out of step, so one's prologue and epilogue hide under the other's key loop (what short key
+// sequences need), and a workgroup is exactly one row of a block mask.
+template <int kW>
+struct WgShape {
+  static_assert(kW == 8 || kW == 4, "workgroups of 8 or 4 waves");
+  static constexpr int kThreads = kW * 64;
+  static constexpr int kRows = kW * 32;                // query rows per workgroup
+  static constexpr int kStages = kW == 8 ? 8 : 4;      // LDS ring (power of two): tiles j-1 .. j+kAhead live at step j
+  static constexpr int kAhead = kW == 8 ? 4 : 2;       // global -> LDS copies are issued this many tiles ahead
+  static constexpr int kCopies = 2 * (8 / kW);         // 1 KiB copy instructions per wave and tile (K and V^T halves)
+  static constexpr int kRingBytes = kStages * 2 * kTileBytes;
+};
 constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f
 constexpr float kMagicF = 12582912.0f;
 constexpr float kPShift = 8.0f;           // P is scaled by 2^8 before the e4m3 cast
 constexpr int kStageBytes = 2 * kTileBytes;  // K tile + V tile
-constexpr int kStages = 8;                   // LDS ring (power of two): tiles j-1 .. j+kAhead live at step j
-constexpr int kAhead = 4;                    // HBM -> LDS copies are issued this many tiles ahead (<= 6)
+constexpr int kSparseMaxKeyTiles4 = 1024;    // 4-wave workgroups keep a shorter tile list so that two fit a compute unit
 constexpr int kMaxKeyTiles = 4096;           // K scales of one head are kept in LDS: Lk <= 262144
+constexpr int kShortKeyTiles = 16;           // dense calls with at most this many key tiles (Lk <= 1024) take 4-wave workgroups
+constexpr int kShortMaxKeyTiles = 2048;      // the most key tiles a dense 4-wave workgroup can hold scales for
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -107,10 +120,14 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
 // kSplit: the workgroup takes one of `p.n_split` equal runs of key tiles of its (head, query block) and leaves
 // unnormalised accumulators, running maxima and row sums in the workspace for sage_attn_merge_kernel.  Used for
 // the workgroups beyond the last full round of the chip, which would otherwise hold it for a whole round alone.
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit>
-__global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg, int n_wg,
-                                                                     int wg_per_xcd) {
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW>
+__global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg,
+                                                                                   int n_wg, int wg_per_xcd) {
   static_assert(!(kSparse && kSplit), "the key split is built for the dense loop only");
+  static_assert(!kSplit || kW == 8, "the key split is built for 256-row workgroups");
+  using Shape = WgShape<kW>;
+  constexpr int kThreadsAttn = Shape::kThreads, kRowsWg = Shape::kRows, kStages = Shape::kStages, kAhead = Shape::kAhead;
+  constexpr int kListMax = kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4;
   int wg, split = 0;
   if constexpr (kSplit) {
     const int item = blockIdx.x / p.n_split;
@@ -134,7 +151,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction: keep it scalar
   const int l32 = lane & 31, hh = lane >> 5;
-  const int q0 = qwg * kAttnQPerWg + wave * 32;
+  const int q0 = qwg * kRowsWg + wave * 32;
   // query rows [0, lq) of this batch take part: all of them, or the caller's per-batch count; the rows from lq up
   // to Lq exist in the output and are written as zeros
   int lq = p.Lq;
@@ -158,7 +175,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     const int per = (tiles + p.n_split - 1) / p.n_split;
     tile0 = split * per;
     const int tile1 = min(tiles, tile0 + per);
-    if (tile0 >= tile1 || qwg * kAttnQPerWg >= lq) {  // nothing in this run (few tiles, a batch entry without keys, or no query row): an empty partial
+    if (tile0 >= tile1 || qwg * kRowsWg >= lq) {  // nothing in this run (few tiles, a batch entry without keys, or no query row): an empty partial
       if (active) {
         const int row = wave * 32 + l32;
         float* po = p.split_o + ((int64_t)blockIdx.x * kAttnQPerWg + row) * kD + 64 * hh;
@@ -170,7 +187,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     }
     lk = min(lk, tile1 * kBlkK) - tile0 * kBlkK;  // from here on the run is the whole key sequence
   } else {
-    if (lk == 0 || qwg * kAttnQPerWg >= lq) {  // no key, or none of the workgroup's rows takes part
+    if (lk == 0 || qwg * kRowsWg >= lq) {  // no key, or none of the workgroup's rows takes part
       write_zero_rows();
       return;
     }
@@ -225,7 +242,6 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
 
   const uint8_t* k_src = reinterpret_cast<const uint8_t*>(p.k_tiles) + ((int64_t)bhk * p.nkb + tile0) * kTileBytes;  // uniform
   const uint8_t* v_src = p.v_tiles + ((int64_t)bhk * p.nkb + tile0) * kTileBytes;
-  const unsigned copy_off = tid * 16;  // this lane's 16 bytes inside a tile
   const float* ks_ptr = p.k_scale + (int64_t)bhk * p.nkb + tile0;
   const int nkb = (lk + kBlkK - 1) / kBlkK;  // tiles this batch uses; p.nkb stays the per-head stride
   // K scales live in LDS behind the ring: a per-tile global load would share the in-order
@@ -241,7 +257,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   // Causal attention (key <= query row) runs through the same list: the workgroup lists the tiles up
   // to the one holding its last row, a wave leaves alone the tiles past its own last row, and the one
   // tile that straddles its rows' diagonal is masked element by element.
-  int* s_list = reinterpret_cast<int*>(smem + kStages * kStageBytes + kSparseMaxKeyTiles * 4);
+  int* s_list = reinterpret_cast<int*>(smem + kStages * kStageBytes + kListMax * 4);
   int n_tiles = nkb;  // loop length: list entries with a mask, key tiles without
   // a wave's 32 rows start at a multiple of 32, so exactly one 64-key tile holds their diagonal
   const int my_last = (kSparse && p.causal) ? (q0 >> 6) : 0x7fffffff;
@@ -249,9 +265,10 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     if (wave == 0) {
       const int nqm = (p.Lq + kMaskBlkQ - 1) / kMaskBlkQ;
       const bool masked = p.block_mask != nullptr;
-      const int8_t* m0 = masked ? p.block_mask + b * p.mask_sB + h * p.mask_sH + (int64_t)(2 * qwg) * p.nkb : nullptr;
-      const bool two = 2 * qwg + 1 < nqm;
-      const int wg_tiles = p.causal ? min(nkb, ((qwg * kAttnQPerWg + kAttnQPerWg - 1) >> 6) + 1) : nkb;
+      constexpr int kMaskRows = kRowsWg / kMaskBlkQ;  // mask rows a workgroup covers: 2 or 1
+      const int8_t* m0 = masked ? p.block_mask + b * p.mask_sB + h * p.mask_sH + (int64_t)(kMaskRows * qwg) * p.nkb : nullptr;
+      const bool two = kMaskRows == 2 && 2 * qwg + 1 < nqm;
+      const int wg_tiles = p.causal ? min(nkb, ((qwg * kRowsWg + kRowsWg - 1) >> 6) + 1) : nkb;
       int base = 0;
       for (int j0 = 0; j0 < wg_tiles; j0 += 64) {
         const int j = j0 + lane;
@@ -266,10 +283,10 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
         if (keep) s_list[base + pre] = j | (f0 << 16) | (f1 << 17);
         base += __popcll(bal);
       }
-      if (lane == 0) s_list[kSparseMaxKeyTiles] = base;
+      if (lane == 0) s_list[kListMax] = base;
     }
     __syncthreads();
-    n_tiles = __builtin_amdgcn_readfirstlane(s_list[kSparseMaxKeyTiles]);
+    n_tiles = __builtin_amdgcn_readfirstlane(s_list[kListMax]);
     if (n_tiles == 0) {  // neither mask row allows any key
       write_zero_rows();
       return;
@@ -286,7 +303,7 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
   auto mine_at = [&](int jj) -> bool {
     if constexpr (kSparse) {
       const int e = __builtin_amdgcn_readfirstlane(s_list[jj]);
-      return ((e >> (16 + (wave >> 2))) & 1) != 0 && (e & 0xffff) <= my_last;
+      return ((e >> (16 + (kW == 8 ? (wave >> 2) : 0))) & 1) != 0 && (e & 0xffff) <= my_last;
     }
     return true;
   };
@@ -334,25 +351,32 @@ __global__ __launch_bounds__(kThreadsAttn) void sage_attn_fwd_kernel(const AttnP
     // clamped: past the end the last tile is copied again into a stage nobody reads any more,
     // which keeps the loop free of branches and the outstanding-copy count constant
     const int jl = tile_of(min(tile, n_tiles - 1));
-    const uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes + wave * 1024;
-    lds_copy16(k_src + (int64_t)jl * kTileBytes, copy_off, dst);
-    lds_copy16(v_src + (int64_t)jl * kTileBytes, copy_off, dst + kTileBytes);
+    const uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes;
+#pragma unroll
+    for (int c = 0; c < 8 / kW; ++c) {  // this wave's 1 KiB slices of the two tiles: slice c * kW + wave
+      const int slice = c * kW + wave;
+      const unsigned off = (unsigned)(slice * 64 + lane) * 16;
+      lds_copy16(k_src + (int64_t)jl * kTileBytes, off, dst + slice * 1024);
+      lds_copy16(v_src + (int64_t)jl * kTileBytes, off, dst + slice * 1024 + kTileBytes);
+    }
   };
   // wait until every copy except those of the newest (kAhead - 2) tiles has landed, then meet
   // the other waves.  Plain s_barrier: a fence here would drain ALL copies and undo the prefetch.
   auto tile_barrier = [&]() {
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * (kAhead - 2)) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Shape::kCopies * (kAhead - 2)) : "memory");
   };
 
   // Every ordinary global load above (Q fragments, scales) must have returned before the first
   // asynchronous copy is issued: the compiler would otherwise drain ALL memory operations,
   // copies included, at the first use of a loaded value inside the loop.
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  // Stage 7's V half is read (times P = 0) by the first loop iteration: make it finite.
-  *reinterpret_cast<uint4*>(smem + (kStages - 1) * kStageBytes + kTileBytes + tid * 16) = make_uint4(0, 0, 0, 0);
+  // The last stage's V half is read (times P = 0) by the first loop iteration: make it finite.
+#pragma unroll
+  for (int c = 0; c < 8 / kW; ++c)
+    *reinterpret_cast<uint4*>(smem + (kStages - 1) * kStageBytes + kTileBytes + (c * kThreadsAttn + tid) * 16) = make_uint4(0, 0, 0, 0);
 #pragma unroll
   for (int t = 0; t < kAhead; ++t) issue_copy(t);
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * (kAhead - 2)) : "memory");  // tiles 0, 1 visible
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(Shape::kCopies * (kAhead - 2)) : "memory");  // tiles 0, 1 visible
 
   if (!active) {
     // same copy / barrier sequence as the active waves
@@ -675,8 +699,15 @@ __global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p
              acc.z * inv_l * s4.z + m4.z * keep_mean, acc.w * inv_l * s4.w + m4.w * keep_mean);
 }
 
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false>
-hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
+// dynamic LDS of one instantiation: tile ring + K scales (+ the tile list and its length with a mask or causal)
+template <bool kSparse, int kW>
+constexpr size_t max_lds() {
+  return kSparse ? WgShape<kW>::kRingBytes + 2 * (kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4) * 4 + 1024
+                 : WgShape<kW>::kRingBytes + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
+}
+
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8>
+hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
   // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
   constexpr int kMaxDevices = 64;
@@ -686,15 +717,24 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, dim3 block, size_t lds
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   if (!requested[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kSparse ? kStages * kStageBytes + 2 * kSparseMaxKeyTiles * 4 + 1024
-                                    : kStages * kStageBytes + kMaxKeyTiles * 4);
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_lds<kSparse, kW>());
     if (e != hipSuccess) return e;
     requested[dev].store(true, std::memory_order_release);
   }
-  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit><<<grid, block, lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
+}
+
+// the four (dtype, exp2 form) instantiations behind one (mask, split, workgroup shape) choice
+template <bool kSparse, bool kSplit, int kW>
+hipError_t launch_shape(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd, hipStream_t s) {
+  const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
+  if (p.exact_exp2)
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
+  return bf16 ? launch_variant<KSANA_SAGE_BF16, true, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+              : launch_variant<KSANA_SAGE_FP16, true, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
 }
 
 // compute units of the current device (the size of one round of workgroups: one workgroup per unit)
@@ -714,6 +754,10 @@ int compute_units() {
 }  // namespace
 
 void plan_key_split(int n_wg, int nkb, int* first_wg, int* runs) {
+  if (nkb <= kShortKeyTiles) {  // these shapes run in 4-wave workgroups, which are never cut
+    *first_wg = n_wg, *runs = 0;
+    return;
+  }
   const int cus = compute_units();
   const int rest = n_wg % cus;
   int n_split = 0;
@@ -725,57 +769,58 @@ void plan_key_split(int n_wg, int nkb, int* first_wg, int* runs) {
   *runs = n_split;
 }
 
+// Workgroup shape for a call: 4-wave workgroups (two per compute unit) when a block mask or causal masking is
+// involved (a workgroup is then one 128-row mask row, so no wave multiplies a tile only the neighbouring mask row
+// asked for) and for short key sequences (a workgroup's fixed costs - operand loads, first copies, the output store -
+// then weigh as much as its key loop and hide under the other workgroup's); 8-wave workgroups otherwise, which copy
+// every K/V tile once per 256 rows instead of once per 128.  p.wg_waves (4 or 8) overrides the choice.
+static int pick_wg_waves(const AttnParams& p) {
+  if (p.wg_waves == 4 || p.wg_waves == 8) return p.wg_waves;
+  const bool sparse = p.block_mask != nullptr || p.causal;
+  if (sparse) return p.nkb <= kSparseMaxKeyTiles4 ? 4 : 8;
+  return p.nkb <= kShortKeyTiles ? 4 : 8;
+}
+
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   if (p.nkb > kMaxKeyTiles) return hipErrorInvalidValue;
+  const bool sparse = p.block_mask != nullptr || p.causal;
+  if (sparse && p.nkb > kSparseMaxKeyTiles) return hipErrorInvalidValue;
+  int waves = pick_wg_waves(p);
+  if (waves == 4 && p.nkb > (sparse ? kSparseMaxKeyTiles4 : kShortMaxKeyTiles)) waves = 8;
+  if (waves == 4) {
+    const int n_qwg = (p.Lq + WgShape<4>::kRows - 1) / WgShape<4>::kRows;
+    const int n_wg = p.B * p.Hq * n_qwg;
+    const int wg_per_xcd = (n_wg + 7) / 8;
+    const dim3 grid(wg_per_xcd * 8);
+    if (sparse) return launch_shape<true, false, 4>(p, grid, max_lds<true, 4>(), n_qwg, n_wg, wg_per_xcd, s);
+    const size_t lds = WgShape<4>::kRingBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
+    return launch_shape<false, false, 4>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
+  }
   const int n_qwg = (p.Lq + kAttnQPerWg - 1) / kAttnQPerWg;
   const int n_wg = p.B * p.Hq * n_qwg;
   const int wg_per_xcd = (n_wg + 7) / 8;
-  const dim3 grid(wg_per_xcd * 8), block(kThreadsAttn);
-  const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
-  if (p.block_mask != nullptr || p.causal) {
-    if (p.nkb > kSparseMaxKeyTiles) return hipErrorInvalidValue;
-    // tile ring + K scales of the listed tiles + the tile list and its length
-    const size_t lds = kStages * kStageBytes + 2 * kSparseMaxKeyTiles * 4 + 1024;
-    if (p.exact_exp2)
-      return bf16 ? launch_variant<KSANA_SAGE_BF16, false, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
-                  : launch_variant<KSANA_SAGE_FP16, false, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, true, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, true, true>(p, grid, block, lds, n_qwg, n_wg, wg_per_xcd, s);
-  }
+  const dim3 grid(wg_per_xcd * 8);
+  if (sparse) return launch_shape<true, false, 8>(p, grid, max_lds<true, 8>(), n_qwg, n_wg, wg_per_xcd, s);
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
-  const size_t lds = kStages * kStageBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
-  auto launch_dense = [&](const AttnParams& pp, dim3 g, int wgs, int per_xcd, bool split) -> hipError_t {
-    if (split) {
-      if (pp.exact_exp2)
-        return bf16 ? launch_variant<KSANA_SAGE_BF16, false, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
-                    : launch_variant<KSANA_SAGE_FP16, false, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
-      return bf16 ? launch_variant<KSANA_SAGE_BF16, true, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
-                  : launch_variant<KSANA_SAGE_FP16, true, false, true>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
-    }
-    if (pp.exact_exp2)
-      return bf16 ? launch_variant<KSANA_SAGE_BF16, false, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
-                  : launch_variant<KSANA_SAGE_FP16, false, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, true, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, true, false>(pp, g, block, lds, n_qwg, wgs, per_xcd, s);
-  };
+  const size_t lds = WgShape<8>::kRingBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
   // The workgroups beyond the last full round of the chip (one workgroup per compute unit) would hold it for a
   // whole round alone.  When they are few, each is cut into runs of key tiles that together fill a round, and a
   // small kernel merges the runs: 2568 workgroups are then 10 rounds and a bit instead of 11, 280 are 1.1 instead of 2.
   int n_full = n_wg, n_split = 0;
   if (p.split_o != nullptr) plan_key_split(n_wg, p.nkb, &n_full, &n_split);
-  if (n_split == 0) return launch_dense(p, grid, n_wg, wg_per_xcd, false);
+  if (n_split == 0) return launch_shape<false, false, 8>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   const int rest = n_wg - n_full;
   if (n_full > 0) {
     const int per_xcd = (n_full + 7) / 8;
-    const hipError_t e = launch_dense(p, dim3(per_xcd * 8), n_full, per_xcd, false);
+    const hipError_t e = launch_shape<false, false, 8>(p, dim3(per_xcd * 8), lds, n_qwg, n_full, per_xcd, s);
     if (e != hipSuccess) return e;
   }
   AttnParams ps = p;
   ps.split_first_wg = n_full;
   ps.n_split = n_split;
-  const hipError_t e = launch_dense(ps, dim3(rest * n_split), n_wg, 0, true);
+  const hipError_t e = launch_shape<false, true, 8>(ps, dim3(rest * n_split), lds, n_qwg, n_wg, 0, s);
   if (e != hipSuccess) return e;
-  if (bf16)
+  if (p.o.dtype == KSANA_SAGE_BF16)
     sage_attn_merge_kernel<KSANA_SAGE_BF16><<<dim3(rest, kAttnQPerWg / 8), dim3(256), 0, s>>>(ps, n_qwg);
   else
     sage_attn_merge_kernel<KSANA_SAGE_FP16><<<dim3(rest, kAttnQPerWg / 8), dim3(256), 0, s>>>(ps, n_qwg);

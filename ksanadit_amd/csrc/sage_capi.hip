@@ -452,7 +452,8 @@ int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_mask(s, block_mask, mask_st)) return rc;
   if (int rc = check_causal(s, causal)) return rc;
-  if (flags & ~KSANA_SAGE_FLAG_PWL_EXP2) return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
+  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_WG_4_WAVES | KSANA_SAGE_FLAG_WG_8_WAVES))
+    return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
   if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
@@ -470,6 +471,7 @@ int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[
   p.split_o = ws_at<float>(ws, l.split_o);
   p.split_ml = ws_at<float>(ws, l.split_ml);
   p.split_first_wg = 0, p.n_split = 0;
+  p.wg_waves = (flags & KSANA_SAGE_FLAG_WG_4_WAVES) ? 4 : ((flags & KSANA_SAGE_FLAG_WG_8_WAVES) ? 8 : 0);
   p.o = ksana_sage::OutTensor{static_cast<uint16_t*>(o), o_st[0], o_st[1], o_st[2], dtype};
   p.B = s->B, p.Hq = s->Hq, p.Hkv = s->Hkv, p.Lq = s->Lq, p.Lk = s->Lk;
   p.lq_pad = l.lq_pad, p.nkb = l.nkb;
@@ -525,7 +527,7 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
   if (int rc = check_tensor("v", v, dtype, v_st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
-  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_SMOOTH_V))
+  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_SMOOTH_V | KSANA_SAGE_FLAG_WG_4_WAVES | KSANA_SAGE_FLAG_WG_8_WAVES))
     return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
   {

@@ -109,6 +109,7 @@ struct AttnParams {
   float* split_o;
   float* split_ml;
   int split_first_wg, n_split;  // filled in by the launcher
+  int wg_waves;  // 0: the launcher picks the workgroup shape; 4 or 8: forced (for measurements and tests)
 };
 constexpr int kMaxSplitPartials = 256;  // (workgroups beyond the last full round) x (runs each) never exceeds this
 constexpr int kMinTilesPerSplit = 8;    // a run shorter than this does not repay its prologue

@@ -307,20 +307,23 @@ def key_split_plan(ws: SageWorkspace):
 
 
 def attn_fwd(ws: SageWorkspace, out: torch.Tensor, causal: bool = False, pwl_exp2: bool = False,
-             k_lens=None, block_mask=None, q_lens=None) -> torch.Tensor:
+             k_lens=None, block_mask=None, q_lens=None, wg_waves: int | None = None) -> torch.Tensor:
     """Attention on the quantized operands in ``ws``.  ``k_lens`` (optional, one int per batch entry): batch ``b``
     attends to keys ``[0, k_lens[b])`` only, the meaning the reference's callers give it (wan_model.py:182-189,
     flash_attn.py:131-139); a batch entry without keys yields zeros.  ``block_mask`` (optional, int8/bool
     ``[B, H, ceil(Lq/128), ceil(Lk/64)]``, leading dims may broadcast): block ``(i, j)`` non-zero lets query rows
     ``128 i ..`` attend to keys ``64 j ..`` - the ``mask_id`` of the reference's block-sparse call
     (radial_sage_attn.py:170-176).  ``q_lens`` (optional, one int per batch entry): only the first ``q_lens[b]`` query
-    rows of batch ``b`` are computed, the rest of the output is zeros (flash_attn.py:120-124 packs exactly those rows)."""
+    rows of batch ``b`` are computed, the rest of the output is zeros (flash_attn.py:120-124 packs exactly those rows).
+    ``wg_waves`` (4 or 8; default: the library's choice) forces the workgroup shape - for measurements and tests."""
     _require_hip(out)
     if out.dim() != 4:
         raise ValueError("out must be [B, Lq, H, D]")
     ws.require(out.device, B=out.shape[0], Lq=out.shape[1], Hq=out.shape[2], D=out.shape[3])
     lib = _capi.load()
-    flags = _capi.FLAG_PWL_EXP2 if pwl_exp2 else 0
+    if wg_waves not in (None, 4, 8):
+        raise ValueError("wg_waves must be 4 or 8")
+    flags = (_capi.FLAG_PWL_EXP2 if pwl_exp2 else 0) | {None: 0, 4: _capi.FLAG_WG_4_WAVES, 8: _capi.FLAG_WG_8_WAVES}[wg_waves]
     kl = _k_lens_arg(k_lens, out.shape[0], out.device)
     ql = _k_lens_arg(q_lens, out.shape[0], out.device, "q_lens")
     s = ws.shape

@@ -506,7 +506,7 @@ def test_v_smoothing_adds_the_mean_back(hip_device, exact):
 
 @pytest.mark.parametrize("exact", [True, False], ids=["exact_exp2", "pwl_exp2"])
 @pytest.mark.parametrize("B,Lq,Lk,Hq,Hkv,dtype,k_lens", [
-    (1, 100, 1000, 2, 2, torch.bfloat16, None),      # 2 query blocks, 16 key tiles -> 2 runs each
+    (1, 100, 1100, 2, 2, torch.bfloat16, None),      # 2 query blocks, 18 key tiles (ragged) -> 2 runs each
     (1, 300, 2100, 3, 1, torch.float16, None),       # 6 blocks, ragged last tile, grouped heads
     (2, 700, 4096, 2, 2, torch.bfloat16, [4096, 1500]),  # per-batch key counts: later runs of batch 1 are empty
     (1, 256, 8192, 1, 1, torch.bfloat16, [0]),       # no keys at all: every run empty, zeros out
@@ -602,6 +602,61 @@ SCHEME_BUDGET = {
 # Full shapes, all heads, per group of 8 heads against torch SDPA on the GPU: worst element over 8 x L x 128 outputs
 # relative to that group's max|O| (the tail of the same int8 effect over 8 - 40 times more rows than above)
 FULL_SIZE_WORST = {"wan14b_480p": 0.20, "wan14b_720p": 0.22, "qwen_cfg": 0.15}
+
+
+def test_wan_cross_attention_at_model_size(hip_device):
+    """WanCrossAttention (wan_model.py:233-251): every one of the 32760 video tokens of the 14B model attends to the
+    512 text tokens (text_len, wan_model.py:546), 40 heads, no rotation, k_lens=None, dense_only=True.  Two heads
+    against the CPU SDPA oracle and the emulation, all heads against torch SDPA on the GPU, through the operator with
+    the kwargs the block passes."""
+    Lq, Lk, H = 32760, 512, 40
+    print(f"cross attention Lq={Lq} Lk={Lk} H={H}", flush=True)
+    g = torch.Generator().manual_seed(4321)
+    q = torch.randn((1, Lq, H, 128), generator=g).to(torch.bfloat16)
+    k = (torch.randn((1, Lk, H, 128), generator=g) * 1.5 + 2.0 * torch.randn((1, 1, H, 128), generator=g)).to(torch.bfloat16)
+    v = torch.randn((1, Lk, H, 128), generator=g).to(torch.bfloat16)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    sage = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN))(num_heads=H, head_size=128)
+    sdpa = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.TORCH_SDPA))(num_heads=H, head_size=128)
+    out = sage(qd, kd, vd, k_lens=None, dense_only=True)
+    assert out.shape == qd.shape and out.dtype == qd.dtype and out.is_contiguous()
+    ref_gpu = sdpa(qd, kd, vd)
+    for h0 in range(0, H, 8):
+        assert _cos(out[:, :, h0 : h0 + 8], ref_gpu[:, :, h0 : h0 + 8]) >= COS_MIN
+    err = (out.float() - ref_gpu.float()).abs()
+    assert err.max().item() <= 0.1 * ref_gpu.float().abs().max().item()
+    ref = sdpa_ref(q[:, :, :2], k[:, :, :2], v[:, :, :2])
+    assert _cos(out[:, :, :2].cpu(), ref) >= COS_MIN
+    two = sage_ops.workspace_for(qd[:, :, :2], kd[:, :, :2])
+    o2 = sage_ops.sageattn(qd[:, :, :2], kd[:, :, :2], vd[:, :, :2], workspace=two).cpu()
+    assert torch.equal(o2, out[:, :, :2].cpu())  # heads are independent
+    emul = _emul_from_ws(two, Lq, Lk, q.dtype)
+    assert (o2.float() - emul.float()).abs().max() <= 2e-2 * emul.float().abs().max()
+    # this shape runs in 4-wave workgroups; 8-wave ones give the same bits (same arithmetic per row)
+    assert torch.equal(sage_ops.attn_fwd(two, torch.empty_like(qd[:, :, :2]), wg_waves=8).cpu(), o2)
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(causal=True), dict(mask=0.5), dict(k_lens=[700, 0, 65])],
+                         ids=["dense", "causal", "mask", "k_lens"])
+def test_both_workgroup_shapes_give_the_same_bits(hip_device, kw):
+    """The kernel comes in workgroups of 8 waves (256 query rows, one per compute unit) and of 4 (128 rows, two per
+    unit); which one runs is the library's choice.  A query row's arithmetic does not depend on it."""
+    B, L, H = 3, 700, 2
+    q, k, v = _rand_qkv(B, L, L, H, H, seed=31)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    sage_ops.sageattn(qd, kd, vd, workspace=ws)
+    args = dict(causal=kw.get("causal", False), k_lens=kw.get("k_lens"))
+    if "mask" in kw:
+        args["block_mask"] = (torch.rand((H, -(-L // 128), -(-L // 64)), generator=torch.Generator().manual_seed(1)) < kw["mask"]).to(torch.int8)
+    a = sage_ops.attn_fwd(ws, torch.empty_like(qd), wg_waves=8, **args).cpu()
+    b = sage_ops.attn_fwd(ws, torch.empty_like(qd), wg_waves=4, **args).cpu()
+    assert torch.isfinite(a.float()).all()
+    if not args["causal"] and "block_mask" not in args:
+        # the 8-wave form cuts the key loop of this small grid into runs and merges them: same attention, other rounding
+        assert (a.float() - b.float()).abs().max() <= 0.08 * a.float().abs().max()
+    else:
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("name", ["wan5b_720p", "wan14b_480p", "wan14b_720p", "qwen_cfg"])
