@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 11
+#define KSANA_SAGE_ABI_VERSION 12
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -173,6 +173,16 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t v_strides[4], con
  * read of V.  smooth_v == 0 is ksana_sage_quant_v. */
 int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[4], const ksana_sage_shape* shape,
                               int smooth_v, void* workspace, void* stream);
+
+/* Block means for the sparse-linear backend's block map: out[b, h, i, :] = mean of x[b, i*rows_per_block : (i+1)*
+ * rows_per_block, h, :] (the last block may be shorter), fp32 sum / number of rows, rounded to x's dtype; out is
+ * [B, H, ceil(L / rows_per_block), D] in x's dtype, contiguous; x is [B, L, H, D] with `strides` like q/k/v (D = 128).
+ * With centre != NULL (device, fp32 [B, H, D]) every x - centre is rounded to x's dtype before it is summed: the
+ * reference pools `k - torch.mean(k, dim=-2, keepdim=True)`, a tensor in k's dtype (sage_sla.py:79-81); the k_mean
+ * area of a workspace after ksana_sage_quant_k holds exactly that mean.  rows_per_block: a multiple of 32, <= 256.
+ * Replaces the Triton kernel compress_kernel / mean_pool (sage_sla.py:43-75). */
+int ksana_sage_block_means(const void* x, int dtype, const int64_t strides[4], int B, int H, int L, int rows_per_block,
+                           const float* centre, void* out, void* stream);
 
 /* Did a workgroup of the last ksana_sage_quant_k / ksana_sage_quant_v on this workspace give up waiting for the
  * others of its head?  Both quantizers read their input once: a workgroup keeps its rows in registers while the

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -32,6 +32,7 @@ EXPORTS = (
     "ksana_sage_attn_fwd",
     "ksana_sage_attn_key_split",
     "ksana_sage_quant_status",
+    "ksana_sage_block_means",
     "ksana_sage_mfma_probe",
     "ksana_sage_forward",
     "ksana_sage_quant_q_prep",
@@ -95,6 +96,8 @@ def _declare(lib):
     ip = C.POINTER(C.c_int)
     lib.ksana_sage_attn_key_split.argtypes, lib.ksana_sage_attn_key_split.restype = [sp, ip, ip], i
     lib.ksana_sage_quant_status.argtypes, lib.ksana_sage_quant_status.restype = [vp, sp, vp, ip, ip], i
+    lib.ksana_sage_block_means.argtypes = [vp, i, st, i, i, i, i, vp, vp, vp]
+    lib.ksana_sage_block_means.restype = i
     lib.ksana_sage_mfma_probe.argtypes = [vp, C.c_uint64, i, i, vp, C.POINTER(C.c_double)]
     lib.ksana_sage_mfma_probe.restype = i
     lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, f, i, i, i, vp, vp]

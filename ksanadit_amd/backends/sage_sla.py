@@ -2,18 +2,19 @@
 
 Drop-in for ksana/operations/attention/backends/sage_sla.py:100-292.  Per call (unless ``dense_only``):
 
-1. a block map: q and the mean-centred k are averaged over blocks of 128 query rows / 64 keys, the block
-   averages are multiplied, and every query block keeps its ``topk`` share of the key blocks with the largest
-   products (sage_sla.py:43-90, 189);
-2. block-sparse quantized attention over the kept blocks (sage_sla.py:196-271) - here this package's masked
-   kernel, which takes the int8 map as it is;
+1. a block map: q and the mean-centred k are averaged over blocks of 128 query rows / 64 keys (the reference's one
+   in-repo GPU kernel, ``compress_kernel`` / ``mean_pool``, sage_sla.py:43-75 - here the HIP kernel behind
+   ``ksana_sage_block_means``, which reads the ``[B, L, H, D]`` tensors as they are and takes k's mean from the
+   quantizer's workspace), the block averages are multiplied, and every query block keeps its ``topk`` share of the key
+   blocks with the largest products (sage_sla.py:78-90, 189);
+2. block-sparse quantized attention over the kept blocks (sage_sla.py:196-271) - this package's masked kernel, which
+   takes the int8 map as it is, on the operands quantized once for both steps;
 3. a linear-attention branch on softmax feature maps of q and k, passed through the block's ``proj_l`` layer, added
    to the sparse result (sage_sla.py:273-287).
 
-Steps 1 and 3 are a handful of dense torch operations and stay torch operations; step 2 is the hot part.
-Block averages are fp32 sums divided by the block's row count, rounded to the input type, as the reference's
-pooling kernel computes them (sage_sla.py:43-63); which of two key blocks with (nearly) equal products makes the
-cut may differ from the reference, whose pooling runs in another summation order.
+The product of the block averages, the top-k selection and the linear branch are a handful of dense torch operations
+(library GEMMs, ``topk``, ``softmax``), as they are in the reference.  Which of two key blocks with equal products
+makes the cut is whatever ``torch.topk`` decides, there as here.
 """
 
 from __future__ import annotations
@@ -21,39 +22,31 @@ from __future__ import annotations
 import torch
 import torch.nn.functional as F
 
-from .. import _capi, platform
+from .. import _capi, platform, sage_ops
 from ..config import KsanaAttentionBackend, KsanaSageSLAConfig
-from ..sage_ops import MASK_BLKK, MASK_BLKQ, block_sparse_sage2_attn
+from ..sage_ops import MASK_BLKK, MASK_BLKQ
 from .base import KsanaAttentionBackendImpl
 
 
-def block_means(x: torch.Tensor, rows: int) -> torch.Tensor:
-    """``[B, H, L, D]`` -> ``[B, H, ceil(L / rows), D]``: mean over each run of ``rows`` positions (the last run may be
-    shorter), accumulated in fp32 and rounded to ``x.dtype``."""
-    B, H, L, D = x.shape
-    nblk = -(-L // rows)
-    pad = nblk * rows - L
-    xf = x.float()
-    if pad:
-        xf = F.pad(xf, (0, 0, 0, pad))
-    sums = xf.view(B, H, nblk, rows, D).sum(dim=3)
-    counts = torch.full((nblk,), float(rows), device=x.device)
-    counts[-1] = rows - pad
-    return (sums / counts.view(1, 1, nblk, 1)).to(x.dtype)
-
-
-def topk_block_map(q: torch.Tensor, k: torch.Tensor, topk_ratio: float, blk_q: int = MASK_BLKQ,
-                   blk_k: int = MASK_BLKK) -> tuple[torch.Tensor, int]:
-    """int8 ``[B, H, ceil(Lq / blk_q), ceil(Lk / blk_k)]`` with ``topk`` ones per row, and ``topk``
-    (``get_block_map``, sage_sla.py:78-90).  q, k are ``[B, H, L, D]``."""
-    centred = k - torch.mean(k, dim=-2, keepdim=True)
-    score = block_means(q, blk_q) @ block_means(centred, blk_k).transpose(-1, -2)
+def block_map_from_pooled(pooled_q: torch.Tensor, pooled_k: torch.Tensor, topk_ratio: float) -> tuple[torch.Tensor, int]:
+    """int8 ``[B, H, nq, nk]`` with ``topk`` ones per row, and ``topk`` (the second half of ``get_block_map``,
+    sage_sla.py:83-90).  ``pooled_*``: block averages ``[B, H, n, D]``, k's taken after centring."""
+    score = pooled_q @ pooled_k.transpose(-1, -2)
     nk = score.shape[-1]
     keep = min(nk, int(topk_ratio * nk))
     picked = torch.topk(score, keep, dim=-1, sorted=False).indices
     block_map = torch.zeros_like(score, dtype=torch.int8)
     block_map.scatter_(-1, picked, 1)
     return block_map, keep
+
+
+def topk_block_map(query: torch.Tensor, key: torch.Tensor, k_mean: torch.Tensor, topk_ratio: float,
+                   blk_q: int = MASK_BLKQ, blk_k: int = MASK_BLKK) -> tuple[torch.Tensor, int]:
+    """``get_block_map`` (sage_sla.py:78-90) for ``[B, L, H, D]`` tensors on a HIP device.  ``k_mean``: fp32
+    ``[B, H, D]``, k's mean over the sequence rounded to k's dtype - what the K quantizer leaves in its workspace."""
+    pooled_q = sage_ops.block_means(query, blk_q)
+    pooled_k = sage_ops.block_means(key, blk_k, centre=k_mean)
+    return block_map_from_pooled(pooled_q, pooled_k, topk_ratio)
 
 
 def linear_branch(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
@@ -103,12 +96,18 @@ class SageSLAAttentionImpl(KsanaAttentionBackendImpl):
     def sla_forward(self, query, key, value, proj_l, return_sparsity: bool = False):
         """``[B, L, H, D]`` in and out; ``proj_l`` is the block's linear layer for the linear branch."""
         dtype = query.dtype
+        if dtype not in (torch.float16, torch.bfloat16):
+            query, key, value = (t.to(torch.bfloat16) for t in (query, key, value))
+        # quantize once; the block map is built next to the quantized operands and drives the attention over them
+        ws = sage_ops.workspace_for(query, key)
+        sage_ops.quant_q(query, ws, query.shape[-1] ** -0.5)
+        sage_ops.quant_k(key, ws, True)
+        sage_ops.quant_v(value, ws)
+        block_map, kept = topk_block_map(query, key, ws.k_mean, self.topk)
+        o_sparse = sage_ops.attn_fwd(ws, torch.empty_like(query), block_mask=block_map)
         q, k, v = (t.transpose(1, 2) for t in (query, key, value))  # [B, H, L, D] views
-        block_map, kept = topk_block_map(q, k, self.topk)
-        o_sparse = block_sparse_sage2_attn(query, key, value, block_map, tensor_layout="NHD",
-                                           sm_scale=q.shape[-1] ** -0.5)
         o_linear = linear_branch(q, k, v)
-        with torch.amp.autocast("cuda", dtype=dtype):
+        with torch.amp.autocast("cuda", dtype=query.dtype):
             o_linear = proj_l(o_linear)
         out = (o_sparse.transpose(1, 2) + o_linear).to(dtype).transpose(1, 2)
         if return_sparsity:

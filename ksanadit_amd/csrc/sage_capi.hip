@@ -426,6 +426,20 @@ int ksana_sage_quant_status(const void* ws, const ksana_sage_shape* s, void* str
   return e == hipSuccess ? 0 : hip_fail(e, "status copy");
 }
 
+int ksana_sage_block_means(const void* x, int dtype, const int64_t st[4], int B, int H, int L, int rows_per_block,
+                           const float* centre, void* out, void* stream) {
+  if (B < 1 || H < 1 || L < 1 || B > 65535 || H > 65535)
+    return fail(KSANA_SAGE_EINVAL, "bad extent (B=%d H=%d L=%d)", B, H, L);
+  if (rows_per_block < 32 || rows_per_block > 256 || rows_per_block % 32 != 0)
+    return fail(KSANA_SAGE_ENOTSUP, "rows_per_block=%d: a multiple of 32 up to 256 is supported", rows_per_block);
+  if (int rc = check_tensor("x", x, dtype, st, B, L, H)) return rc;
+  if (!out || (reinterpret_cast<uintptr_t>(out) & 1u)) return fail(KSANA_SAGE_EINVAL, "out is null or misaligned");
+  if (reinterpret_cast<uintptr_t>(centre) & 3u) return fail(KSANA_SAGE_EINVAL, "centre is not 4-byte aligned");
+  hipError_t e = ksana_sage::launch_block_means(in_tensor(x, dtype, st), B, H, L, rows_per_block, centre,
+                                                static_cast<uint16_t*>(out), static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? 0 : hip_fail(e, "block means launch");
+}
+
 int ksana_sage_attn_key_split(const ksana_sage_shape* s, int* first_workgroup, int* runs) {
   if (int rc = check_shape(s)) return rc;
   if (!first_workgroup || !runs) return fail(KSANA_SAGE_EINVAL, "out-pointer is null");

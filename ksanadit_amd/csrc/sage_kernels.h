@@ -86,6 +86,11 @@ hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb,
                                 float* v_inv, float* v_mean, uint8_t* v_tiles, const QuantSync& sync, hipStream_t s,
                                 bool* used);
 
+// out[b, h, blk, :] = mean of the rows of block blk (rows per block: a multiple of 32, at most 256) of x[b, :, h, :],
+// of round_to_half(x - centre[b, h, :]) when centre != nullptr; out is [B, H, ceil(L / rows), 128] in x's half type
+hipError_t launch_block_means(const InTensor& x, int B, int H, int L, int rows, const float* centre, uint16_t* out,
+                              hipStream_t s);
+
 struct AttnParams {
   const int8_t* q_i8;
   const float* q_scale;

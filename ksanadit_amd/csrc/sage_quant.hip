@@ -1036,6 +1036,67 @@ __global__ __launch_bounds__(kThreads) void quant_v_fused_kernel(const uint16_t*
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Block means: out[b, h, blk, d] = mean over the rows [blk * rows, min((blk + 1) * rows, L)) of x[b, :, h, d],
+// optionally of x - centre[b, h, d] with each difference rounded to the tensor's half type first (the reference
+// forms `k - mean(k)` as a half tensor before it pools it).  fp32 sum in a frozen order - row r of the block goes to
+// slot r % 32, a slot adds its rows in increasing order, the 32 slots meet in an adjacent-pair tree - divided by the
+// number of rows that exist and rounded to the half type.  One workgroup per block; rows <= 256, a multiple of 32.
+// grid = (nblk, H, B).
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kThreads) void block_mean_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
+                                                              int64_t sH, int H, int L, int rows,
+                                                              const float* __restrict__ centre,
+                                                              uint16_t* __restrict__ out) {
+  const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const uint16_t* base = x + b * sB + h * sH + c16 * 16;
+  const int64_t bh = (int64_t)b * H + h;
+  float cen[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) cen[e] = centre != nullptr ? centre[bh * kD + c16 * 16 + e] : 0.0f;
+  float acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+  for (int i = 0; i < rows / kSlots; ++i) {
+    const int row = blk * rows + i * kSlots + slot;
+    float v[16];
+    load_row16<DT>(base + (int64_t)row * sL, row < L, v);
+    if (centre != nullptr && row < L) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) v[e] = through_half<DT>(v[e] - cen[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = i == 0 ? v[e] : acc[e] + v[e];
+  }
+#pragma unroll
+  for (int m = 8; m <= 32; m <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = acc[e] + __shfl_xor(acc[e], m);
+  }
+  __shared__ float s_w[4][kD];
+  const int wave = t >> 6, lane = t & 63;
+  if (lane < 8) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
+  }
+  __syncthreads();
+  if (t < kD) {
+    const float sum = (s_w[0][t] + s_w[1][t]) + (s_w[2][t] + s_w[3][t]);
+    const float n = (float)min(rows, L - blk * rows);
+    const float mean = __fdiv_rn(sum, n);
+    const int64_t nblk = gridDim.x;
+    uint16_t bits;
+    if constexpr (DT == KSANA_SAGE_BF16) {
+      bits = __builtin_bit_cast(uint16_t, (__bf16)mean);
+    } else {
+      bits = __builtin_bit_cast(uint16_t, (_Float16)mean);
+    }
+    out[(bh * nblk + blk) * kD + t] = bits;
+  }
+}
+
 __global__ void clear_ints_kernel(int* p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -1169,6 +1230,13 @@ int resident_workgroups(K kernel, size_t lds) {
 constexpr long long kWaitLimitTicks = 200000000;  // 2 s of the 100 MHz wall clock
 
 }  // namespace
+
+hipError_t launch_block_means(const InTensor& x, int B, int H, int L, int rows, const float* centre, uint16_t* out,
+                              hipStream_t s) {
+  const dim3 grid((L + rows - 1) / rows, H, B), block(kThreads);
+  KSANA_DISPATCH_DT(x.dtype, (block_mean_kernel<DT><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, rows, centre, out)));
+  return hipGetLastError();
+}
 
 hipError_t launch_clear_ints(int* p, int n, hipStream_t s) {
   if (n <= 0) return hipSuccess;

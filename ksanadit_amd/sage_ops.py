@@ -256,6 +256,27 @@ def quant_v(v: torch.Tensor, ws: SageWorkspace, smooth_v: bool = False) -> None:
     _capi.check(rc, "ksana_sage_quant_v")
 
 
+def block_means(x: torch.Tensor, rows: int, centre: torch.Tensor | None = None) -> torch.Tensor:
+    """``[B, L, H, D]`` -> ``[B, H, ceil(L / rows), D]`` in ``x.dtype``: the mean of every run of ``rows`` positions (the
+    last may be shorter), fp32 sum / count; with ``centre`` (fp32 ``[B, H, D]``) of ``x - centre`` rounded to ``x.dtype``
+    first.  The pooling of the reference's ``mean_pool`` (sage_sla.py:43-75) on the layout the blocks hand over."""
+    _require_hip(x)
+    if x.dim() != 4 or x.shape[3] != 128:
+        raise ValueError("block_means expects [B, L, H, 128]")
+    x = _usable(x)
+    B, L, H, D = x.shape
+    if centre is not None:
+        if centre.shape != (B, H, D) or centre.dtype != torch.float32 or centre.device != x.device:
+            raise ValueError(f"centre must be float32 [{B}, {H}, {D}] on {x.device}")
+        centre = centre.contiguous()
+    out = torch.empty((B, H, -(-L // rows), D), dtype=x.dtype, device=x.device)
+    rc = _capi.load().ksana_sage_block_means(x.data_ptr(), _DTYPES[x.dtype], _strides(x), B, H, L, rows,
+                                             None if centre is None else centre.data_ptr(), out.data_ptr(),
+                                             _stream_ptr(x.device))
+    _capi.check(rc, "ksana_sage_block_means")
+    return out
+
+
 def quant_status(ws: SageWorkspace) -> tuple[int, int]:
     """``(k_status, v_status)`` of the last K / V quantization on ``ws``: 0, or 1 when a workgroup gave up waiting for
     the others of its head (see ``ksana_sage_quant_status``).  Synchronises the current stream; for tests."""

@@ -372,32 +372,76 @@ def test_radial_backend_gates_and_masks(hip_device):
         op(qd, kd, vd, step_iter=7, block_id=5, k_lens=two, latent_shape=[1, 16, frames, 32, 32])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,H,rows", [(1, 64, 1, 64), (2, 130, 3, 64), (1, 1000, 2, 128), (1, 257, 4, 128), (1, 96, 1, 32)])
+def test_block_means_kernel_bit_exact(hip_device, B, L, H, rows, dtype):
+    """The HIP counterpart of the reference's pooling kernel (compress_kernel / mean_pool, sage_sla.py:43-75) against
+    the oracle's frozen-order restatement: plain, centred with a per-channel offset (the ``k - mean(k)`` the reference
+    pools), and on a strided view."""
+    from oracle.sla_ref import block_means_ref
+
+    print(f"case block means B={B} L={L} H={H} rows={rows} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(L * 3 + H)
+    x = (torch.randn((B, L, H, 128), generator=g) * 2.0 + torch.randn((1, 1, H, 128), generator=g)).to(dtype)
+    c = torch.randn((B, H, 128), generator=g)
+    xd = x.to(hip_device)
+    assert torch.equal(sage_ops.block_means(xd, rows).cpu(), block_means_ref(x.permute(0, 2, 1, 3), rows))
+    assert torch.equal(sage_ops.block_means(xd, rows, centre=c.to(hip_device)).cpu(),
+                       block_means_ref(x.permute(0, 2, 1, 3), rows, centre=c))
+    fused = torch.randn((B, L, 3, H, 128), generator=g).to(dtype)
+    view = fused.to(hip_device)[:, :, 1]
+    assert not view.is_contiguous()
+    assert torch.equal(sage_ops.block_means(view, rows).cpu(), block_means_ref(fused[:, :, 1].permute(0, 2, 1, 3), rows))
+    with pytest.raises(NotImplementedError):
+        sage_ops.block_means(xd, 48)
+
+
 def test_sla_backend_sparse_plus_linear(hip_device):
     """sage_sla.py:141-292: dense when asked, else block-sparse attention on the top-k map plus the projected
-    linear branch."""
+    linear branch.  The map, the linear branch and the composition are checked against the oracle's own restatements
+    (oracle/sla_ref.py), not against the backend's helpers."""
     from ksanadit_amd.backends.sage_sla import linear_branch, topk_block_map
     from ksanadit_amd.config import KsanaSageSLAConfig
+    from oracle.sla_ref import block_map_ref, linear_branch_ref
 
     B, L, H = 1, 1024, 2
     q, k, v = _rand_qkv(B, L, L, H, H, seed=81)
+    # give the key blocks distinct levels along a direction the queries lean towards, so that the top-k cut is clear
+    g = torch.Generator().manual_seed(82)
+    direction = torch.randn(128, generator=g)
+    direction /= direction.norm()
+    level = torch.randperm(L // 64, generator=g).float().repeat_interleave(64)  # one level per 64-key block
+    k = (k.float() + 0.6 * level[None, :, None, None] * direction).to(torch.bfloat16)
+    q = (q.float() + 2.0 * direction).to(torch.bfloat16)
     qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
     op = pick_attn_op(KsanaSageSLAConfig(topk=0.25))(num_heads=H, head_size=128, causal=False)
     proj = torch.nn.Linear(128, 128, bias=False).to(hip_device).to(torch.bfloat16)
     torch.nn.init.normal_(proj.weight, std=0.05)
     assert torch.equal(op(qd, kd, vd, dense_only=True, proj_l=proj).cpu(), sage_ops.sageattn(qd, kd, vd).cpu())
     with torch.no_grad():
-        out = op(qd, kd, vd, proj_l=proj).cpu()
+        out = op(qd, kd, vd, proj_l=proj)
+        again, sparsity = op._attn_impl.sla_forward(qd, kd, vd, proj, return_sparsity=True)
+    assert torch.equal(out, again) and sparsity == 0.25
+    out = out.cpu()
     assert out.shape == q.shape and out.dtype == q.dtype
-    # the same composition from the oracle's masked SDPA and torch on the CPU
-    qt, kt, vt = (t.transpose(1, 2) for t in (q, k, v))
-    bmap, kept = topk_block_map(qd.transpose(1, 2), kd.transpose(1, 2), 0.25)
-    assert kept == 4 and (bmap.sum(dim=-1) == 4).all()
-    sparse_ref = sdpa_ref(q, k, v, block_mask=bmap.cpu())
+    # the block map: the oracle's restatement of get_block_map, on inputs where the cut is unambiguous
+    want_map, kept, gap = block_map_ref(q, k, 0.25)
+    assert kept == 4 and float(gap.min()) > 0.1, "the test inputs must leave no near-tie at the cut"
+    ws = sage_ops.workspace_for(qd, kd)
+    sage_ops.quant_k(kd, ws, True)
+    got_map, got_kept = topk_block_map(qd, kd, ws.k_mean, 0.25)
+    assert got_kept == kept and torch.equal(got_map.cpu(), want_map)
+    # the linear branch: the backend's torch composition on the GPU against the oracle's on the CPU
+    lin_gpu = linear_branch(*(t.transpose(1, 2) for t in (qd, kd, vd))).cpu()
+    lin_ref = linear_branch_ref(q, k, v)
+    assert _cos(lin_gpu, lin_ref) >= 0.9999
+    assert (lin_gpu.float() - lin_ref.float()).abs().max() <= 0.03 * lin_ref.float().abs().max()
+    # the composition: masked SDPA oracle on the oracle's map + the projected oracle branch
     with torch.no_grad():
-        lin = proj.cpu().float()(linear_branch(qt.float(), kt.float(), vt.float())).transpose(1, 2)
-    ref = sparse_ref.float() + lin
-    assert _cos(out, ref) >= 0.998
-    assert (out.float() - ref).abs().max() <= 0.15 * max(ref.abs().max().item(), 0.1)
+        lin = proj.cpu().float()(lin_ref.float()).transpose(1, 2)
+    ref = sdpa_ref(q, k, v, block_mask=want_map).float() + lin
+    assert _cos(out, ref) >= COS_MIN
+    assert (out.float() - ref).abs().max() <= 0.1 * max(ref.abs().max().item(), 0.1)
 
 
 def test_forward_replays_from_a_hip_graph(hip_device):
