@@ -86,7 +86,7 @@ __device__ __forceinline__ void pin(T& x) {
 }
 
 template <int DT>
-__device__ __forceinline__ void store4(uint16_t* dst, float a, float b, float c, float d) {
+__device__ __forceinline__ uint2 half4(float a, float b, float c, float d) {
   uint32_t lo, hi;
   if constexpr (DT == KSANA_SAGE_BF16) {
     typedef __bf16 b2 __attribute__((ext_vector_type(2)));
@@ -99,7 +99,11 @@ __device__ __forceinline__ void store4(uint16_t* dst, float a, float b, float c,
     lo = __builtin_bit_cast(uint32_t, x);
     hi = __builtin_bit_cast(uint32_t, y);
   }
-  *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+  return make_uint2(lo, hi);
+}
+template <int DT>
+__device__ __forceinline__ void store4(uint16_t* dst, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(dst) = half4<DT>(a, b, c, d);
 }
 
 // S^T tile (64 keys x 32 queries) of one wave: two 32-key sub-tiles, four 32-channel steps.
@@ -246,7 +250,9 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   const int nkb = (lk + kBlkK - 1) / kBlkK;  // tiles this batch uses; p.nkb stays the per-head stride
   // K scales live in LDS behind the ring: a per-tile global load would share the in-order
   // vmcnt queue with the tile copies and stall on all of them
-  float* s_ks = reinterpret_cast<float*>(smem + kStages * kStageBytes);
+  // behind the ring: the head's V scales and V means (2 x 128 floats, read by the epilogue), then its K scales
+  float* s_vs = reinterpret_cast<float*>(smem + kStages * kStageBytes);
+  float* s_ks = s_vs + 2 * kD;
 
   // ---- block mask: the workgroup's list of key tiles ---------------------------------------
   // A mask row covers 128 query rows, a workgroup two of them (waves 0-3, waves 4-7).  Wave 0
@@ -257,7 +263,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // Causal attention (key <= query row) runs through the same list: the workgroup lists the tiles up
   // to the one holding its last row, a wave leaves alone the tiles past its own last row, and the one
   // tile that straddles its rows' diagonal is masked element by element.
-  int* s_list = reinterpret_cast<int*>(smem + kStages * kStageBytes + kListMax * 4);
+  int* s_list = reinterpret_cast<int*>(s_ks + kListMax);
   int n_tiles = nkb;  // loop length: list entries with a mask, key tiles without
   // a wave's 32 rows start at a multiple of 32, so exactly one 64-key tile holds their diagonal
   const int my_last = (kSparse && p.causal) ? (q0 >> 6) : 0x7fffffff;
@@ -295,6 +301,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   } else {
     for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
   }
+  if (tid < 2 * kD) s_vs[tid] = tid < kD ? p.v_scale[(int64_t)bhk * kD + tid] : p.v_mean[(int64_t)bhk * kD + tid - kD];
   // key tile behind loop position jj, and whether this wave's mask row asks for it
   auto tile_of = [&](int jj) -> int {
     if constexpr (kSparse) return __builtin_amdgcn_readfirstlane(s_list[jj]) & 0xffff;
@@ -633,30 +640,40 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     if (hh == 0) reinterpret_cast<float2*>(p.split_ml)[(int64_t)blockIdx.x * kAttnQPerWg + row] = make_float2(m_run, lacc[0]);
     return;
   }
-  // ---- epilogue: O = O^T / rowsum * v_scale, written [B, Lq, H, D] ----------------------
+  // ---- epilogue: O = O^T / rowsum * v_scale (+ the V mean), written [B, Lq, H, D] ---------------
+  // A lane holds its query row in pieces of four channels; stored as they are, every store instruction would
+  // touch 32 rows with 16 bytes each.  The rows go through LDS instead (the tile ring is free once every wave is
+  // past its last tile) and leave as whole 256-byte rows, 16 bytes per lane.
   const int q = q0 + l32;
   // zero for a mask row that allows none of its keys (an empty sum, not 0/0) and for rows at or beyond lq
   const float inv_l = ((!kSparse || lacc[0] > 0.0f) && q < lq) ? 1.0f / lacc[0] : 0.0f;
-  if (q < p.Lq) {
-    uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
-    const float* vs = p.v_scale + (int64_t)bhk * kD;
-    // the channel means the V quantizer took off come back here (rows of P sum to one); they are zeros
-    // without V smoothing, and a row that saw no key stays zero
-    const float* vm = p.v_mean + (int64_t)bhk * kD;
-    const float keep_mean = inv_l != 0.0f ? 1.0f : 0.0f;
+  // the channel means the V quantizer took off come back here (rows of P sum to one); they are zeros without V
+  // smoothing, and a row that saw no key stays zero
+  const float keep_mean = inv_l != 0.0f ? 1.0f : 0.0f;
+  constexpr int kPitch = 2 * kD + 16;  // bytes per staged row: 16 bytes of padding spread the rows over the banks
+  __syncthreads();  // waves that ended early (no query rows) do not count
+  uint8_t* stage = smem + wave * (32 * kPitch);
+  const float4* vs4 = reinterpret_cast<const float4*>(s_vs);
+  const float4* vm4 = reinterpret_cast<const float4*>(s_vs + kD);
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) {
+  for (int dt = 0; dt < 4; ++dt) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int d = 32 * dt + 8 * g + 4 * hh;
-        const float4 s4 = *reinterpret_cast<const float4*>(vs + d);
-        const float4 m4 = *reinterpret_cast<const float4*>(vm + d);
-        store4<DT>(orow + d, oacc[dt][4 * g + 0] * inv_l * s4.x + m4.x * keep_mean,
-                   oacc[dt][4 * g + 1] * inv_l * s4.y + m4.y * keep_mean,
-                   oacc[dt][4 * g + 2] * inv_l * s4.z + m4.z * keep_mean,
-                   oacc[dt][4 * g + 3] * inv_l * s4.w + m4.w * keep_mean);
-      }
+    for (int g = 0; g < 4; ++g) {
+      const int d = 32 * dt + 8 * g + 4 * hh;
+      const float4 s4 = vs4[d >> 2];
+      const float4 m4 = vm4[d >> 2];
+      *reinterpret_cast<uint2*>(stage + l32 * kPitch + 2 * d) =
+          half4<DT>(oacc[dt][4 * g + 0] * inv_l * s4.x + m4.x * keep_mean, oacc[dt][4 * g + 1] * inv_l * s4.y + m4.y * keep_mean,
+                    oacc[dt][4 * g + 2] * inv_l * s4.z + m4.z * keep_mean, oacc[dt][4 * g + 3] * inv_l * s4.w + m4.w * keep_mean);
     }
+  }
+  // LDS serves one wave's accesses in order: the reads below see the writes above
+  uint16_t* obase = p.o.ptr + b * p.o.sB + h * p.o.sH;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int idx = i * 64 + lane, r = idx >> 4, c = idx & 15;  // row r of the wave, 16-byte piece c of it
+    const uint4 piece = *reinterpret_cast<const uint4*>(stage + r * kPitch + 16 * c);
+    if (q0 + r < p.Lq) *reinterpret_cast<uint4*>(obase + (int64_t)(q0 + r) * p.o.sL + 8 * c) = piece;
   }
 }
 
@@ -702,8 +719,8 @@ __global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p
 // dynamic LDS of one instantiation: tile ring + K scales (+ the tile list and its length with a mask or causal)
 template <bool kSparse, int kW>
 constexpr size_t max_lds() {
-  return kSparse ? WgShape<kW>::kRingBytes + 2 * (kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4) * 4 + 1024
-                 : WgShape<kW>::kRingBytes + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
+  return kSparse ? WgShape<kW>::kRingBytes + 1024 + 2 * (kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4) * 4 + 1024
+                 : WgShape<kW>::kRingBytes + 1024 + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
 }
 
 template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8>
@@ -793,7 +810,7 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
     const int wg_per_xcd = (n_wg + 7) / 8;
     const dim3 grid(wg_per_xcd * 8);
     if (sparse) return launch_shape<true, false, 4>(p, grid, max_lds<true, 4>(), n_qwg, n_wg, wg_per_xcd, s);
-    const size_t lds = WgShape<4>::kRingBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
+    const size_t lds = WgShape<4>::kRingBytes + 1024 + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
     return launch_shape<false, false, 4>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   }
   const int n_qwg = (p.Lq + kAttnQPerWg - 1) / kAttnQPerWg;
@@ -802,7 +819,7 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const dim3 grid(wg_per_xcd * 8);
   if (sparse) return launch_shape<true, false, 8>(p, grid, max_lds<true, 8>(), n_qwg, n_wg, wg_per_xcd, s);
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
-  const size_t lds = WgShape<8>::kRingBytes + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
+  const size_t lds = WgShape<8>::kRingBytes + 1024 + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
   // The workgroups beyond the last full round of the chip (one workgroup per compute unit) would hold it for a
   // whole round alone.  When they are few, each is cut into runs of key tiles that together fill a round, and a
   // small kernel merges the runs: 2568 workgroups are then 10 rounds and a bit instead of 11, 280 are 1.1 instead of 2.
