@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 12
+#define KSANA_SAGE_ABI_VERSION 13
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -119,7 +119,24 @@ typedef struct ksana_sage_prep {
   const int32_t* grid_sizes;   /* HOST array [B, 3]: (frames, height, width) per batch entry; the        */
                                /* reference reads it on the host as well (rope.py:107).  Needed with     */
                                /* rope_freqs; B <= 16; each extent <= rope_rows; F*H*W <= L              */
+  /* kind == KSANA_SAGE_PREP_QWEN: what QwenDoubleStreamAttention.forward does to the joint q and k (text rows
+   * first, image rows behind them, qwen/attention.py:340-357) instead of the Wan steps above:
+   *   RMSNorm over the D channels of every head (norm_q / norm_k for the image rows, norm_added_q / norm_added_k for
+   *     the text rows; float_rmsnorm of ops.py:62-72 with the statistic per head), then
+   *   apply_rotary_emb_qwen (qwen/attention.py:31-59): pairs (x[2i], x[2i+1]) times one complex64 factor per
+   *     (row, pair), image rows from rope_freqs_img, text rows from rope_freqs_txt.
+   * q_norm_weight / k_norm_weight are then the IMAGE weights, fp32 [D]; the fields below the text side.  The caller
+   * hands over the raw projections already concatenated (text first) - the concatenation the block performs anyway.
+   * NULL weights skip the norm of that segment, NULL tables its rotation.  rope_freqs / grid_sizes are not used. */
+  int32_t kind;                    /* KSANA_SAGE_PREP_WAN (0) or KSANA_SAGE_PREP_QWEN (2)                     */
+  int32_t txt_len;                 /* rows [0, txt_len) are text, [txt_len, L) image                          */
+  const float* q_norm_weight_txt;  /* device, fp32 [D], 16-byte aligned, or NULL                              */
+  const float* k_norm_weight_txt;
+  const float* rope_freqs_txt;     /* device, complex64 [txt_len, D/2] as (re, im), 16-byte aligned, or NULL  */
+  const float* rope_freqs_img;     /* device, complex64 [L - txt_len, D/2]                                    */
 } ksana_sage_prep;
+#define KSANA_SAGE_PREP_WAN 0
+#define KSANA_SAGE_PREP_QWEN 2
 
 /* Library identity.  No counterpart in the reference. */
 int ksana_sage_abi_version(void);

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -19,6 +19,7 @@ FLAG_PWL_EXP2 = 1
 FLAG_SMOOTH_V = 2
 FLAG_WG_4_WAVES = 4
 FLAG_WG_8_WAVES = 8
+PREP_WAN, PREP_QWEN = 0, 2
 
 EXPORTS = (
     "ksana_sage_abi_version",
@@ -69,6 +70,12 @@ class Prep(C.Structure):
         ("rope_rows", C.c_int32),
         ("rope_freqs", C.c_void_p),
         ("grid_sizes", C.POINTER(C.c_int32)),
+        ("kind", C.c_int32),
+        ("txt_len", C.c_int32),
+        ("q_norm_weight_txt", C.c_void_p),
+        ("k_norm_weight_txt", C.c_void_p),
+        ("rope_freqs_txt", C.c_void_p),
+        ("rope_freqs_img", C.c_void_p),
     ]
 
 

@@ -164,9 +164,35 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
 int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name, const int64_t st[4], int B, int L,
               float* inv_rms, ksana_sage::PrepParams* pp, const ksana_sage::PrepParams** out) {
   *out = nullptr;
-  if (!prep || (!weight && !prep->rope_freqs)) return 0;
+  if (!prep) return 0;
+  if (prep->kind != KSANA_SAGE_PREP_WAN && prep->kind != KSANA_SAGE_PREP_QWEN)
+    return fail(KSANA_SAGE_EINVAL, "prep kind %d unknown", prep->kind);
+  if (prep->kind == KSANA_SAGE_PREP_QWEN) {
+    const bool is_q = name[0] == 'q';
+    const float* w_txt = is_q ? prep->q_norm_weight_txt : prep->k_norm_weight_txt;
+    if (!weight && !w_txt && !prep->rope_freqs_txt && !prep->rope_freqs_img) return 0;
+    memset(pp, 0, sizeof(*pp));
+    pp->L = L;
+    pp->kind = 2;
+    if (prep->txt_len < 0 || prep->txt_len > L)
+      return fail(KSANA_SAGE_EINVAL, "txt_len=%d outside [0, %s length %d]", prep->txt_len, name, L);
+    if (!(prep->norm_eps >= 0.0f)) return fail(KSANA_SAGE_EINVAL, "norm_eps must be >= 0");
+    const void* ptrs[4] = {weight, w_txt, prep->rope_freqs_txt, prep->rope_freqs_img};
+    for (const void* ptr : ptrs)
+      if (reinterpret_cast<uintptr_t>(ptr) & 15u) return fail(KSANA_SAGE_EINVAL, "%s: a prep pointer is not 16-byte aligned", name);
+    pp->txt_len = prep->txt_len;
+    pp->eps = prep->norm_eps;
+    pp->weight_img = weight;
+    pp->weight_txt = w_txt;
+    pp->freqs_txt = reinterpret_cast<const float2*>(prep->rope_freqs_txt);
+    pp->freqs_img = reinterpret_cast<const float2*>(prep->rope_freqs_img);
+    *out = pp;
+    return 0;
+  }
+  if (!weight && !prep->rope_freqs) return 0;
   memset(pp, 0, sizeof(*pp));
   pp->L = L;
+  pp->kind = 1;
   if (weight) {
     if (reinterpret_cast<uintptr_t>(weight) & 15u)
       return fail(KSANA_SAGE_EINVAL, "%s norm weight not 16-byte aligned", name);
@@ -310,8 +336,9 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
     e = ksana_sage::launch_row_inv_rms(kt, s->B, s->Hkv, s->Lk, prep->norm_eps, ws_at<float>(ws, l.k_rms), hs);
     if (e != hipSuccess) return hip_fail(e, "k row statistic launch");
   }
-  if (one_read('k')) {
-    // one read of K: chunk sums, the head's mean and the quantization in one kernel, when the shape suits it
+  if (one_read('k') || ppp != nullptr) {
+    // one read of K: chunk sums, the head's mean and the quantization in one kernel, when the shape suits it (always
+    // tried when the step before attention is applied on the way in: the rotation is then done once, not twice)
     e = ksana_sage::launch_clear_ints(sync_words, ksana_sage::sync_words(bhk), hs);
     if (e != hipSuccess) return hip_fail(e, "k counter clear launch");
     bool used = false;

@@ -39,6 +39,17 @@ struct PrepParams {
   const float* weight;   // [H * 128] fp32 norm weight
   const double* freqs;   // [rows, 64] complex128 as (re, im); nullptr = no rotation
   int L;
+  // kind 2, the Qwen-Image block (qwen/attention.py:340-353): RMSNorm over the 128 channels of every head (the
+  // statistic is taken inside the kernel), one weight vector for the text rows [0, txt_len) and one for the image rows
+  // behind them, then a rotation by one complex64 factor per (row, pair) from a table per segment.  A nullptr weight
+  // / table switches that step off for its segment.
+  int kind;  // 1: the Wan block (fields above and below), 2: the Qwen block (fields here)
+  int txt_len;
+  float eps;
+  const float* weight_txt;    // [128]
+  const float* weight_img;    // [128]
+  const float2* freqs_txt;    // [txt_len, 64] (re, im)
+  const float2* freqs_img;    // [L - txt_len, 64]
   int grid[kMaxPrepBatch][3];  // (frames, height, width) per batch entry
   // Capacity (table rows) of the per-workgroup LDS copy of the rotation factors, filled in by the
   // launcher for its kernel's rows per workgroup; lds_frames == 0: read `freqs` directly.

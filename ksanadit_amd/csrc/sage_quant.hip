@@ -136,9 +136,59 @@ __device__ __forceinline__ int small_div(int n, int d, int* rem) {
   return q;
 }
 
+template <int M>
+__device__ __forceinline__ float lane_xor(float v);
+
+// The Qwen-Image block's step before attention on the 16 channels [16*c16, 16*c16+16) of one head of token `row`
+// (the 8 lanes c16 = 0..7 of the row are adjacent):
+//   y = half( (x * r) * weight[ch] ),  r = 1 / sqrt(mean_{128 channels}(x^2) + eps)
+//       mean: every lane adds its 16 squares in channel order, the 8 lane sums meet in an adjacent-pair tree
+//   (y[2i], y[2i+1]) -> half( (y[2i] + i*y[2i+1]) * freqs[row, i] )    complex64: four products, one subtraction and
+//       one addition, each rounded to fp32
+template <int DT>
+__device__ __forceinline__ void prep16_qwen(float* x, const PrepParams& pp, int row, int c16) {
+  const bool txt = row < pp.txt_len;
+  const float* w = txt ? pp.weight_txt : pp.weight_img;
+  if (w != nullptr) {
+    float ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) ss = e == 0 ? x[0] * x[0] : ss + x[e] * x[e];  // squares of half values are exact
+    ss = ss + lane_xor<1>(ss);
+    ss = ss + lane_xor<2>(ss);
+    ss = ss + lane_xor<4>(ss);
+    const float r = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(ss, (float)kD) + pp.eps));
+    const float4* w4 = reinterpret_cast<const float4*>(w + c16 * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float4 wj = w4[j];
+      x[4 * j + 0] = through_half<DT>((x[4 * j + 0] * r) * wj.x);
+      x[4 * j + 1] = through_half<DT>((x[4 * j + 1] * r) * wj.y);
+      x[4 * j + 2] = through_half<DT>((x[4 * j + 2] * r) * wj.z);
+      x[4 * j + 3] = through_half<DT>((x[4 * j + 3] * r) * wj.w);
+    }
+  }
+  const float2* tab = txt ? pp.freqs_txt : pp.freqs_img;
+  if (tab != nullptr) {
+    const float4* t4 = reinterpret_cast<const float4*>(tab + (int64_t)(txt ? row : row - pp.txt_len) * (kD / 2) + c16 * 8);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float4 cs = t4[j];  // two factors: (re, im), (re, im)
+      const float a0 = x[4 * j], b0 = x[4 * j + 1], a1 = x[4 * j + 2], b1 = x[4 * j + 3];
+      x[4 * j + 0] = through_half<DT>(a0 * cs.x - b0 * cs.y);
+      x[4 * j + 1] = through_half<DT>(a0 * cs.y + b0 * cs.x);
+      x[4 * j + 2] = through_half<DT>(a1 * cs.z - b1 * cs.w);
+      x[4 * j + 3] = through_half<DT>(a1 * cs.w + b1 * cs.z);
+    }
+  }
+}
+
 template <int DT>
 __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const RopeLds& rl, int b, int row, int h,
                                        int c16) {
+  if (pp.kind == 2) {  // uniform
+    prep16_qwen<DT>(x, pp, row, c16);
+    return;
+  }
   if (pp.inv_rms != nullptr) {
     const float r = pp.inv_rms[(int64_t)b * pp.L + row];
     const float4* w4 = reinterpret_cast<const float4*>(pp.weight + h * kD + c16 * 16);
@@ -1119,7 +1169,7 @@ __global__ void clear_ints_kernel(int* p, int n) {
 // a workgroup; returns the dynamic LDS bytes (0: the kernel reads the table directly).
 static size_t plan_rope_lds(PrepParams* pp, int B, int rows_per_wg) {
   pp->lds_frames = pp->lds_heights = pp->lds_widths = 0;
-  if (pp->freqs == nullptr) return 0;
+  if (pp->kind == 2 || pp->freqs == nullptr) return 0;
   int nf = 0, nh = 0, nw = 0;
   for (int b = 0; b < B; ++b) {
     const int gh = pp->grid[b][1], gw = pp->grid[b][2];

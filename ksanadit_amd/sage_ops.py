@@ -200,6 +200,59 @@ class WanPrep:
         return c, keep
 
 
+@dataclass
+class QwenPrep:
+    """What ``QwenDoubleStreamAttention.forward`` does to q and k before its joint attention call
+    (ksana/models/qwen/attention.py:340-357), handed to the quantizer to apply while it reads them.  q and k are the
+    raw projections of the text tokens followed by those of the image tokens (the concatenation the block performs
+    anyway, here done before instead of after): RMSNorm over the ``D`` channels of every head - ``norm_q`` /
+    ``norm_k`` weights (``[D]``) for the image rows, ``norm_added_q`` / ``norm_added_k`` for the first ``txt_len`` rows -
+    then ``apply_rotary_emb_qwen`` with the complex64 tables ``img_freqs`` ``[L - txt_len, D/2]`` and ``txt_freqs``
+    ``[txt_len, D/2]``.  ``None`` weights skip the norm of that segment, ``None`` tables its rotation."""
+
+    txt_len: int
+    q_norm_weight: torch.Tensor | None = None
+    k_norm_weight: torch.Tensor | None = None
+    q_norm_weight_txt: torch.Tensor | None = None
+    k_norm_weight_txt: torch.Tensor | None = None
+    eps: float = 1e-6
+    img_freqs: torch.Tensor | None = None
+    txt_freqs: torch.Tensor | None = None
+
+    def to_c(self, device):
+        keep = []
+
+        def weight(w):
+            if w is None:
+                return None
+            w = w.to(device=device, dtype=torch.float32).contiguous()
+            if w.numel() != 128:
+                raise ValueError("Qwen norm weights are per head channel: 128 values")
+            keep.append(w)
+            return w.data_ptr()
+
+        def table(t, rows):
+            if t is None:
+                return None
+            if t.dim() != 2 or not t.is_complex() or t.shape[1] != 64:
+                raise ValueError("rotary tables must be complex [rows, 64]")
+            if t.shape[0] < rows:
+                raise ValueError(f"rotary table has {t.shape[0]} rows, the segment {rows}")
+            t = torch.view_as_real(t.to(device=device, dtype=torch.complex64).contiguous())
+            keep.append(t)
+            return t.data_ptr()
+
+        c = _capi.Prep()
+        c.kind = _capi.PREP_QWEN
+        c.txt_len = int(self.txt_len)
+        c.norm_eps = float(self.eps)
+        c.q_norm_weight, c.k_norm_weight = weight(self.q_norm_weight), weight(self.k_norm_weight)
+        c.q_norm_weight_txt, c.k_norm_weight_txt = weight(self.q_norm_weight_txt), weight(self.k_norm_weight_txt)
+        c.rope_freqs_txt = table(self.txt_freqs, self.txt_len)
+        c.rope_freqs_img = table(self.img_freqs, 0)  # its length is checked against L by the caller
+        return c, keep
+
+
 def _as_heads(x: torch.Tensor, num_heads: int | None) -> torch.Tensor:
     """``[B, L, H*D]`` projection -> ``[B, L, H, D]`` view (4-D tensors pass through)."""
     if x.dim() == 4:
@@ -215,7 +268,13 @@ def workspace_for(q: torch.Tensor, k: torch.Tensor) -> SageWorkspace:
     return SageWorkspace.allocate(B, Hq, Hkv, Lq, Lk, D, q.device)
 
 
-def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: WanPrep | None = None) -> None:
+def _check_qwen_rows(prep, L: int) -> None:
+    """The image table of a ``QwenPrep`` must cover the rows behind the text rows."""
+    if isinstance(prep, QwenPrep) and prep.img_freqs is not None and prep.img_freqs.shape[0] < L - prep.txt_len:
+        raise ValueError(f"img_freqs has {prep.img_freqs.shape[0]} rows, the image segment {L - prep.txt_len}")
+
+
+def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: "WanPrep | QwenPrep | None" = None) -> None:
     _require_hip(q)
     ws.require(q.device, B=q.shape[0], Lq=q.shape[1], Hq=q.shape[2], D=q.shape[3])
     q = _usable(q)
@@ -224,13 +283,14 @@ def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: WanPrep |
         rc = lib.ksana_sage_quant_q(q.data_ptr(), _DTYPES[q.dtype], _strides(q), C.byref(ws.shape), sm_scale, ws.ptr,
                                     _stream_ptr(q.device))
     else:
+        _check_qwen_rows(prep, q.shape[1])
         c_prep, _keep = prep.to_c(q.device)
         rc = lib.ksana_sage_quant_q_prep(q.data_ptr(), _DTYPES[q.dtype], _strides(q), C.byref(ws.shape),
                                          C.byref(c_prep), sm_scale, ws.ptr, _stream_ptr(q.device))
     _capi.check(rc, "ksana_sage_quant_q")
 
 
-def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: WanPrep | None = None) -> None:
+def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: "WanPrep | QwenPrep | None" = None) -> None:
     _require_hip(k)
     ws.require(k.device, B=k.shape[0], Lk=k.shape[1], Hkv=k.shape[2], D=k.shape[3])
     k = _usable(k)
@@ -239,6 +299,7 @@ def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: Wan
         rc = lib.ksana_sage_quant_k(k.data_ptr(), _DTYPES[k.dtype], _strides(k), C.byref(ws.shape), int(smooth_k),
                                     ws.ptr, _stream_ptr(k.device))
     else:
+        _check_qwen_rows(prep, k.shape[1])
         c_prep, _keep = prep.to_c(k.device)
         rc = lib.ksana_sage_quant_k_prep(k.data_ptr(), _DTYPES[k.dtype], _strides(k), C.byref(ws.shape),
                                          C.byref(c_prep), int(smooth_k), ws.ptr, _stream_ptr(k.device))
@@ -442,6 +503,9 @@ def sageattn(
         )
         _capi.check(rc, "ksana_sage_forward_masked")
         return out.transpose(1, 2) if tensor_layout == "HND" else out
+    if prep is not None:
+        _check_qwen_rows(prep, Lq)
+        _check_qwen_rows(prep, k.shape[1])
     c_prep, _keep = (None, None) if prep is None else prep.to_c(q.device)
     rc = lib.ksana_sage_forward_prep(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],

@@ -121,3 +121,74 @@ def wan_prep_ref(x: torch.Tensor, weight, eps: float, grid_sizes, freqs, num_hea
     y = x if weight is None else rmsnorm_ref(x, weight, eps)
     y = y.view(B, L, num_heads, HD // num_heads)
     return y if freqs is None else rope_ref(y, grid_sizes, freqs)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The Qwen-Image block's step before attention (ksana/models/qwen/attention.py:340-357):
+#   img_q = norm_q(img_q); txt_q = norm_added_q(txt_q)          RMSNorm over the D channels of every head (:269-272)
+#   x = apply_rotary_emb_qwen(x, freqs)  (:31-59)                complex64: view_as_complex(x.float()) * freqs
+#   joint = cat([txt, img], dim=1)                               text rows first (:355-357)
+# ``RMSNorm.float_rmsnorm`` (ops.py:62-72) is the arithmetic restated; the order of the sum of squares over the 128
+# channels is frozen here: eight accumulators take 16 consecutive channels each, in channel order, and meet in an
+# adjacent-pair tree.  The rotation is written in real arithmetic - four products, one subtraction, one addition, each
+# rounded to fp32 - which is bit for bit what torch's complex64 multiplication computes on the CPU (pinned in
+# tests/test_prep_oracle.py against ``torch.view_as_complex(...) * freqs``, the reference's own expression).
+# ---------------------------------------------------------------------------------------------------------------
+def head_mean_square_ref(x: torch.Tensor) -> torch.Tensor:
+    """fp32 ``mean(x^2)`` over a last dim of 128 in the frozen order described above."""
+    assert x.shape[-1] == 128
+    sq = (x.float() * x.float()).reshape(*x.shape[:-1], 8, 16)  # exact for half inputs
+    acc = sq[..., 0]
+    for e in range(1, 16):
+        acc = acc + sq[..., e]
+    width = 8
+    while width > 1:
+        acc = acc.reshape(*acc.shape[:-1], width // 2, 2)
+        acc = acc[..., 0] + acc[..., 1]
+        width //= 2
+    return acc[..., 0] / torch.tensor(128.0, dtype=torch.float32)
+
+
+def head_rmsnorm_ref(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``[..., 128]`` half in, same out: ``float_rmsnorm`` per head (ops.py:62-72)."""
+    t = (head_mean_square_ref(x) + torch.tensor(eps, dtype=torch.float32)).numpy()
+    r = torch.from_numpy((np.float32(1.0) / np.sqrt(t)).astype(np.float32))[..., None]
+    return ((x.float() * r) * weight.float()).type_as(x)
+
+
+def qwen_rope_ref(x: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+    """``apply_rotary_emb_qwen`` (qwen/attention.py:31-59, one GPU): ``x`` ``[B, L, H, D]``, ``freqs`` complex64
+    ``[>= L, D/2]``; same shape and dtype out."""
+    L = x.shape[1]
+    f = torch.view_as_real(freqs[:L].to(torch.complex64))  # [L, D/2, 2]
+    c, s = f[..., 0][None, :, None, :], f[..., 1][None, :, None, :]
+    xf = x.float().reshape(*x.shape[:-1], -1, 2)
+    a, b = xf[..., 0], xf[..., 1]
+    re = a * c - b * s
+    im = a * s + b * c
+    return torch.stack([re, im], dim=-1).flatten(3).type_as(x)
+
+
+def qwen_prep_ref(x: torch.Tensor, txt_len: int, weight_img, weight_txt, eps: float, img_freqs, txt_freqs) -> torch.Tensor:
+    """The joint ``[B, L, H, D]`` projection (text rows first) -> normed and rotated, ready for attention.
+    ``None`` weights / tables skip that step for their segment."""
+    txt, img = x[:, :txt_len], x[:, txt_len:]
+    if weight_txt is not None:
+        txt = head_rmsnorm_ref(txt, weight_txt, eps)
+    if weight_img is not None:
+        img = head_rmsnorm_ref(img, weight_img, eps)
+    if txt_freqs is not None and txt.shape[1]:
+        txt = qwen_rope_ref(txt, txt_freqs)
+    if img_freqs is not None and img.shape[1]:
+        img = qwen_rope_ref(img, img_freqs)
+    return torch.cat([txt, img], dim=1)
+
+
+def qwen_rope_table(rows: int, axes_dim=(16, 56, 56), theta: float = 10000.0, offset: int = 0) -> torch.Tensor:
+    """A complex64 ``[rows, 64]`` table of the shape ``QwenEmbedRope`` produces (qwen/attention.py:62-96): per axis
+    ``exp(i * pos * theta^(-2j/dim))`` in fp32, the three axes side by side; here every axis simply counts the row."""
+    parts = []
+    for dim in axes_dim:
+        fr = torch.outer(torch.arange(offset, offset + rows).float(), 1.0 / torch.pow(theta, torch.arange(0, dim, 2).float().div(dim)))
+        parts.append(torch.polar(torch.ones_like(fr), fr))
+    return torch.cat(parts, dim=1)

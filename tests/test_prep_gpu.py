@@ -6,7 +6,7 @@ import torch
 
 from ksanadit_amd import sage_ops
 from ksanadit_amd.layout import untile_k
-from ksanadit_amd.sage_ops import WanPrep
+from ksanadit_amd.sage_ops import QwenPrep, WanPrep
 from oracle import prep_ref as pr
 from oracle import quant_ref as qr
 from oracle.sdpa_ref import sdpa_ref
@@ -105,6 +105,64 @@ def test_prep_at_model_row_width_and_length(hip_device):
     assert torch.equal(ws.q_rms.cpu(), pr.inv_rms_ref(qp, 1e-6))
     _check_q(ws, pr.wan_prep_ref(qp, wq, 1e-6, grids, table, H), 128**-0.5, L)
     _check_k(ws, pr.wan_prep_ref(kp, wk, 1e-6, grids, table, H), L)
+
+
+@pytest.mark.parametrize(
+    "B,txt,img,H,dtype,norm,rope",
+    [
+        (1, 7, 50, 2, torch.bfloat16, True, True),
+        (2, 256, 4096, 4, torch.bfloat16, True, True),   # the Qwen-Image 1024 x 1024 joint sequence, CFG pair
+        (2, 33, 300, 3, torch.float16, True, True),
+        (1, 0, 130, 2, torch.bfloat16, True, True),      # no text rows at all
+        (1, 64, 64, 2, torch.bfloat16, True, False),
+        (1, 64, 64, 2, torch.bfloat16, False, True),
+    ],
+)
+def test_quantizer_with_qwen_prep_is_bit_exact(hip_device, B, txt, img, H, dtype, norm, rope):
+    """Per-head RMSNorm (text and image weights) + apply_rotary_emb_qwen on the way into the quantizer
+    (qwen/attention.py:340-357) against the oracle's restatement followed by the plain quantizer oracle."""
+    print(f"case qwen prep B={B} txt={txt} img={img} H={H} {dtype} norm={norm} rope={rope}", flush=True)
+    L = txt + img
+    g = torch.Generator().manual_seed(txt * 7 + img)
+    q = (1.5 * torch.randn((B, L, H, 128), generator=g)).to(dtype)
+    k = (1.5 * torch.randn((B, L, H, 128), generator=g) + 0.7 * torch.randn((1, 1, H, 128), generator=g)).to(dtype)
+    q[:, :txt] *= 3.0  # text tokens of another scale, as in the measured workload
+    w = [(1.0 + 0.2 * torch.randn(128, generator=g)).float() for _ in range(4)]
+    f_img, f_txt = pr.qwen_rope_table(img + 5, offset=-3), pr.qwen_rope_table(max(txt, 1), offset=2000)
+    prep = QwenPrep(txt_len=txt, q_norm_weight=w[0] if norm else None, k_norm_weight=w[1] if norm else None,
+                    q_norm_weight_txt=w[2] if norm else None, k_norm_weight_txt=w[3] if norm else None, eps=1e-6,
+                    img_freqs=f_img if rope else None, txt_freqs=f_txt if rope else None)
+    qd, kd = q.to(hip_device), k.to(hip_device)
+    ws = sage_ops.workspace_for(qd, kd)
+    ws.blob.fill_(0x7F)
+    sage_ops.quant_q(qd, ws, 128**-0.5, prep=prep)
+    sage_ops.quant_k(kd, ws, prep=prep)
+    torch.cuda.synchronize()
+    assert sage_ops.quant_status(ws)[0] == 0
+    q_ref = pr.qwen_prep_ref(q, txt, w[0] if norm else None, w[2] if norm else None, 1e-6, f_img if rope else None, f_txt if rope else None)
+    k_ref = pr.qwen_prep_ref(k, txt, w[1] if norm else None, w[3] if norm else None, 1e-6, f_img if rope else None, f_txt if rope else None)
+    _check_q(ws, q_ref, 128**-0.5, L)
+    _check_k(ws, k_ref, L)
+
+
+def test_qwen_block_path_equals_attention_on_prepared_tensors(hip_device):
+    B, txt, img, H = 2, 40, 500, 3
+    L = txt + img
+    g = torch.Generator().manual_seed(99)
+    q, k, v = ((1.5 * torch.randn((B, L, H, 128), generator=g)).to(torch.bfloat16) for _ in range(3))
+    w = [(1.0 + 0.2 * torch.randn(128, generator=g)).float() for _ in range(4)]
+    f_img, f_txt = pr.qwen_rope_table(img), pr.qwen_rope_table(txt, offset=3000)
+    prep = QwenPrep(txt, w[0], w[1], w[2], w[3], 1e-6, f_img, f_txt)
+    fused = sage_ops.sageattn(q.to(hip_device), k.to(hip_device), v.to(hip_device), prep=prep).cpu()
+    q_ref = pr.qwen_prep_ref(q, txt, w[0], w[2], 1e-6, f_img, f_txt)
+    k_ref = pr.qwen_prep_ref(k, txt, w[1], w[3], 1e-6, f_img, f_txt)
+    plain = sage_ops.sageattn(q_ref.to(hip_device), k_ref.to(hip_device), v.to(hip_device)).cpu()
+    assert torch.equal(fused, plain)
+    a, b = fused.double().flatten(), sdpa_ref(q_ref, k_ref, v).double().flatten()
+    assert float((a @ b) / (a.norm() * b.norm())) >= 0.999
+    with pytest.raises(ValueError, match="rows"):
+        sage_ops.sageattn(q.to(hip_device), k.to(hip_device), v.to(hip_device),
+                          prep=QwenPrep(txt, w[0], w[1], w[2], w[3], 1e-6, f_img[:100], f_txt))
 
 
 def test_prep_argument_errors(hip_device):

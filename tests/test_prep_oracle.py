@@ -167,3 +167,68 @@ def test_wan_prep_composes_norm_then_rope():
     assert out.shape == (1, 12, 2, 128)
     assert torch.equal(out, pr.rope_ref(pr.rmsnorm_ref(x, w, 1e-6).view(1, 12, 2, 128), [(1, 3, 4)], table))
     assert torch.equal(pr.wan_prep_ref(x, None, 0.0, None, None, 2), x.view(1, 12, 2, 128))
+
+
+# ----------------------------------------------------------------------------- the Qwen-Image block (qwen/attention.py:340-357)
+def test_qwen_head_norm_against_scalar_replay_library_routine_and_float64():
+    x = _half((1, 5, 3, 128), 21) * 2.0
+    w = (1.0 + 0.2 * torch.randn(128, generator=torch.Generator().manual_seed(22))).float()
+    got = pr.head_rmsnorm_ref(x, w, 1e-6)
+    assert got.shape == x.shape and got.dtype == x.dtype
+    # scalar replay of the frozen order: 8 accumulators x 16 channels in order, adjacent-pair tree
+    ms = pr.head_mean_square_ref(x)
+    f32 = lambda v: torch.tensor(v, dtype=torch.float32)
+    for t in range(5):
+        for h in range(3):
+            accs = []
+            for c in range(8):
+                a = None
+                for e in range(16):
+                    v = x[0, t, h, 16 * c + e].float()
+                    a = v * v if a is None else a + v * v
+                accs.append(a)
+            while len(accs) > 1:
+                accs = [accs[2 * i] + accs[2 * i + 1] for i in range(len(accs) // 2)]
+            assert ms[0, t, h] == accs[0] / f32(128.0)
+    # the library routine behind torch.nn.RMSNorm (another summation order): equal except for rare last-place flips
+    lib = torch.nn.functional.rms_norm(x.float(), (128,), w, 1e-6).type_as(x)
+    assert (got != lib).float().mean() <= 1e-3
+    assert (got.float() - lib.float()).abs().max() <= 2.0**-7 * lib.float().abs().max()
+    # float64 brute force
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(dim=-1, keepdim=True) + 1e-6) * w.double()
+    assert (got.double() - want).abs().max() <= 2.0**-8 * want.abs().max() + 1e-6
+
+
+def test_qwen_rope_is_torchs_complex64_product_and_a_rotation():
+    x = _half((2, 40, 3, 128), 23) * 1.5
+    table = pr.qwen_rope_table(64, offset=-7)  # negative positions occur in the model's tables too (scale_rope)
+    y = pr.qwen_rope_ref(x, table)
+    # the reference's own expression (qwen/attention.py:37,57-59)
+    xr = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
+    want = torch.view_as_real(xr * table[:40].unsqueeze(1)).flatten(3).type_as(x)
+    assert torch.equal(y, want)
+    # a rotation: pair lengths survive (to bf16 rounding); the row with angle 0 is the identity
+    n_in = x.double().reshape(2, 40, 3, 64, 2).norm(dim=-1)
+    n_out = y.double().reshape(2, 40, 3, 64, 2).norm(dim=-1)
+    assert ((n_in - n_out).abs() <= 2.0**-7 * n_in + 1e-6).all()
+    assert torch.equal(y[:, 7], x[:, 7])  # position -7 + 7 = 0
+    # one pair by hand: axis 0 has dim 16, pair j turns by pos * theta^(-2j/16)
+    pos, j = 5, 3
+    ang = (pos - 7) * 10000.0 ** (-2.0 * j / 16.0)
+    a, b = x[1, pos, 2, 2 * j].double().item(), x[1, pos, 2, 2 * j + 1].double().item()
+    hand = torch.tensor([a * math.cos(ang) - b * math.sin(ang), a * math.sin(ang) + b * math.cos(ang)])
+    assert (y[1, pos, 2, 2 * j : 2 * j + 2].double() - hand).abs().max() <= 2.0**-7 * hand.abs().max() + 1e-6
+
+
+def test_qwen_prep_composes_the_two_streams():
+    g = torch.Generator().manual_seed(24)
+    x = _half((1, 30, 2, 128), 25)
+    w_img, w_txt = (1.0 + 0.1 * torch.randn(128, generator=g)).float(), (1.0 + 0.1 * torch.randn(128, generator=g)).float()
+    f_img, f_txt = pr.qwen_rope_table(20), pr.qwen_rope_table(10, offset=100)
+    out = pr.qwen_prep_ref(x, 10, w_img, w_txt, 1e-6, f_img, f_txt)
+    txt = pr.qwen_rope_ref(pr.head_rmsnorm_ref(x[:, :10], w_txt, 1e-6), f_txt)
+    img = pr.qwen_rope_ref(pr.head_rmsnorm_ref(x[:, 10:], w_img, 1e-6), f_img)
+    assert torch.equal(out, torch.cat([txt, img], dim=1))
+    assert torch.equal(pr.qwen_prep_ref(x, 10, None, None, 0.0, None, None), x)
+    assert torch.equal(pr.qwen_prep_ref(x, 0, w_img, None, 1e-6, None, None), pr.head_rmsnorm_ref(x, w_img, 1e-6))
