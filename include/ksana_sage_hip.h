@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 13
+#define KSANA_SAGE_ABI_VERSION 14
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -128,14 +128,21 @@ typedef struct ksana_sage_prep {
    * q_norm_weight / k_norm_weight are then the IMAGE weights, fp32 [D]; the fields below the text side.  The caller
    * hands over the raw projections already concatenated (text first) - the concatenation the block performs anyway.
    * NULL weights skip the norm of that segment, NULL tables its rotation.  rope_freqs / grid_sizes are not used. */
-  int32_t kind;                    /* KSANA_SAGE_PREP_WAN (0) or KSANA_SAGE_PREP_QWEN (2)                     */
+  int32_t kind;                    /* KSANA_SAGE_PREP_WAN (0), _WAN_COMFY (1), _QWEN (2)                   */
   int32_t txt_len;                 /* rows [0, txt_len) are text, [txt_len, L) image                          */
   const float* q_norm_weight_txt;  /* device, fp32 [D], 16-byte aligned, or NULL                              */
   const float* k_norm_weight_txt;
   const float* rope_freqs_txt;     /* device, complex64 [txt_len, D/2] as (re, im), 16-byte aligned, or NULL  */
   const float* rope_freqs_img;     /* device, complex64 [L - txt_len, D/2]                                    */
+  /* kind == KSANA_SAGE_PREP_WAN_COMFY: the Wan block with rope_func == "comfy" (wan_model.py:169-171): the norm as
+   * for KSANA_SAGE_PREP_WAN, then apply_comfyui_rope (utils/rope.py:180-212): out[2i+e] = m[e][0]*x[2i] +
+   * m[e][1]*x[2i+1] in fp32 with the 2x2 matrix of (row, pair i).  rope_rows is the table's row count here; rows at or
+   * past it are left as they are (the identity padding of rope.py:133-148).  rope_freqs / grid_sizes are not used. */
+  const float* rope_matrices;      /* device, fp32 [rope_rows, D/2, 2, 2]: the `freqs_cis` of EmbedND            */
+                                   /* (rope.py:165-177) without its broadcast dims, 16-byte aligned, or NULL     */
 } ksana_sage_prep;
 #define KSANA_SAGE_PREP_WAN 0
+#define KSANA_SAGE_PREP_WAN_COMFY 1
 #define KSANA_SAGE_PREP_QWEN 2
 
 /* Library identity.  No counterpart in the reference. */

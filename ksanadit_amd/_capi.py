@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -19,7 +19,7 @@ FLAG_PWL_EXP2 = 1
 FLAG_SMOOTH_V = 2
 FLAG_WG_4_WAVES = 4
 FLAG_WG_8_WAVES = 8
-PREP_WAN, PREP_QWEN = 0, 2
+PREP_WAN, PREP_WAN_COMFY, PREP_QWEN = 0, 1, 2
 
 EXPORTS = (
     "ksana_sage_abi_version",
@@ -76,6 +76,7 @@ class Prep(C.Structure):
         ("k_norm_weight_txt", C.c_void_p),
         ("rope_freqs_txt", C.c_void_p),
         ("rope_freqs_img", C.c_void_p),
+        ("rope_matrices", C.c_void_p),
     ]
 
 

@@ -165,7 +165,7 @@ int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name
               float* inv_rms, ksana_sage::PrepParams* pp, const ksana_sage::PrepParams** out) {
   *out = nullptr;
   if (!prep) return 0;
-  if (prep->kind != KSANA_SAGE_PREP_WAN && prep->kind != KSANA_SAGE_PREP_QWEN)
+  if (prep->kind != KSANA_SAGE_PREP_WAN && prep->kind != KSANA_SAGE_PREP_WAN_COMFY && prep->kind != KSANA_SAGE_PREP_QWEN)
     return fail(KSANA_SAGE_EINVAL, "prep kind %d unknown", prep->kind);
   if (prep->kind == KSANA_SAGE_PREP_QWEN) {
     const bool is_q = name[0] == 'q';
@@ -189,10 +189,11 @@ int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name
     *out = pp;
     return 0;
   }
-  if (!weight && !prep->rope_freqs) return 0;
+  const bool comfy = prep->kind == KSANA_SAGE_PREP_WAN_COMFY;
+  if (!weight && !(comfy ? (const void*)prep->rope_matrices : (const void*)prep->rope_freqs)) return 0;
   memset(pp, 0, sizeof(*pp));
   pp->L = L;
-  pp->kind = 1;
+  pp->kind = comfy ? 3 : 1;
   if (weight) {
     if (reinterpret_cast<uintptr_t>(weight) & 15u)
       return fail(KSANA_SAGE_EINVAL, "%s norm weight not 16-byte aligned", name);
@@ -203,7 +204,15 @@ int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name
     pp->inv_rms = inv_rms;
     pp->weight = weight;
   }
-  if (prep->rope_freqs) {
+  if (comfy) {
+    if (prep->rope_matrices) {
+      if (reinterpret_cast<uintptr_t>(prep->rope_matrices) & 15u)
+        return fail(KSANA_SAGE_EINVAL, "rope_matrices not 16-byte aligned");
+      if (prep->rope_rows < 1) return fail(KSANA_SAGE_EINVAL, "rope_rows must be positive");
+      pp->rot = reinterpret_cast<const float4*>(prep->rope_matrices);
+      pp->rot_rows = prep->rope_rows;
+    }
+  } else if (prep->rope_freqs) {
     if (reinterpret_cast<uintptr_t>(prep->rope_freqs) & 15u)
       return fail(KSANA_SAGE_EINVAL, "rope_freqs not 16-byte aligned");
     if (!prep->grid_sizes) return fail(KSANA_SAGE_EINVAL, "rope_freqs given without grid_sizes");

@@ -43,7 +43,10 @@ struct PrepParams {
   // statistic is taken inside the kernel), one weight vector for the text rows [0, txt_len) and one for the image rows
   // behind them, then a rotation by one complex64 factor per (row, pair) from a table per segment.  A nullptr weight
   // / table switches that step off for its segment.
-  int kind;  // 1: the Wan block (fields above and below), 2: the Qwen block (fields here)
+  int kind;  // 1: the Wan block (fields above and below), 2: the Qwen block (fields here), 3: the Wan block with
+             // the rotation given as one 2x2 fp32 matrix per (row, pair) (`rot`, utils/rope.py:180-212)
+  const float4* rot;  // kind 3: [rot_rows, 64] matrices (m00, m01, m10, m11); rows from rot_rows on are not rotated
+  int rot_rows;
   int txt_len;
   float eps;
   const float* weight_txt;    // [128]

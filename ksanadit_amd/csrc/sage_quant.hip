@@ -201,6 +201,21 @@ __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const Rop
       x[4 * j + 3] = through_half<DT>((x[4 * j + 3] * r) * w.w);
     }
   }
+  if (pp.kind == 3) {  // uniform
+    // apply_comfyui_rope (utils/rope.py:180-212): out[2i+e] = m[e][0] * x[2i] + m[e][1] * x[2i+1] in fp32, the first
+    // product rounded on its own, the second fused into the sum (what torch's mul followed by addcmul_ computes)
+    if (pp.rot != nullptr && row < pp.rot_rows) {
+      const float4* m4 = pp.rot + (int64_t)row * (kD / 2) + c16 * 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float4 m = m4[j];
+        const float a = x[2 * j], bb = x[2 * j + 1];
+        x[2 * j] = through_half<DT>(__fmaf_rn(m.y, bb, __fmul_rn(m.x, a)));
+        x[2 * j + 1] = through_half<DT>(__fmaf_rn(m.w, bb, __fmul_rn(m.z, a)));
+      }
+    }
+    return;
+  }
   if (pp.freqs != nullptr) {
     const int gh = pp.grid[b][1], gw = pp.grid[b][2];
     const int plane = gh * gw;

@@ -163,13 +163,19 @@ class WanPrep:
     RMSNorm over the whole token row with fp32 weights (``norm_q.weight`` / ``norm_k.weight``; ``None`` skips it),
     then ``apply_default_rope(x, grid_sizes, freqs)`` (ksana/utils/rope.py:61-128; ``freqs=None`` skips it, as in
     the cross-attention block).  ``freqs`` is the model's complex128 buffer ``[1024, D/2]``, ``grid_sizes`` one
-    ``(frames, height, width)`` per batch entry."""
+    ``(frames, height, width)`` per batch entry.
+
+    With ``rope_func == "comfy"`` (wan_model.py:169-171) the block rotates with ``apply_comfyui_rope``
+    (ksana/utils/rope.py:180-212) instead: pass its ``freqs_cis`` as ``comfy_freqs`` - fp32 2x2 matrices,
+    ``[1, rows, 1, D/2, 2, 2]`` or ``[rows, D/2, 2, 2]`` - and leave ``freqs`` / ``grid_sizes`` unset; token rows past
+    the table are left unrotated (the identity padding of rope.py:133-148)."""
 
     q_norm_weight: torch.Tensor | None = None
     k_norm_weight: torch.Tensor | None = None
     eps: float = 1e-6
     freqs: torch.Tensor | None = None
     grid_sizes: object = None
+    comfy_freqs: torch.Tensor | None = None
 
     def to_c(self, device):
         """The C struct plus the objects that must outlive the call."""
@@ -185,6 +191,18 @@ class WanPrep:
         c = _capi.Prep()
         c.q_norm_weight, c.k_norm_weight = weight(self.q_norm_weight), weight(self.k_norm_weight)
         c.norm_eps = float(self.eps)
+        if self.comfy_freqs is not None:
+            if self.freqs is not None:
+                raise ValueError("give either freqs (default rope) or comfy_freqs, not both")
+            m = self.comfy_freqs
+            if m.dim() == 6 and m.shape[0] == 1 and m.shape[2] == 1:
+                m = m[0, :, 0]
+            if m.dim() != 4 or tuple(m.shape[1:]) != (64, 2, 2) or m.is_complex():
+                raise ValueError(f"comfy_freqs must be [1, rows, 1, 64, 2, 2] or [rows, 64, 2, 2], got {tuple(self.comfy_freqs.shape)}")
+            m = m.to(device=device, dtype=torch.float32).contiguous()
+            keep.append(m)
+            c.kind = _capi.PREP_WAN_COMFY
+            c.rope_matrices, c.rope_rows = m.data_ptr(), m.shape[0]
         if self.freqs is not None:
             if self.freqs.dim() != 2 or not self.freqs.is_complex():
                 raise ValueError("freqs must be a complex [rows, D/2] tensor")

@@ -192,3 +192,46 @@ def qwen_rope_table(rows: int, axes_dim=(16, 56, 56), theta: float = 10000.0, of
         fr = torch.outer(torch.arange(offset, offset + rows).float(), 1.0 / torch.pow(theta, torch.arange(0, dim, 2).float().div(dim)))
         parts.append(torch.polar(torch.ones_like(fr), fr))
     return torch.cat(parts, dim=1)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The Wan block with ``rope_func == "comfy"`` (wan_model.py:169-171): ``EmbedND`` (ksana/utils/rope.py:151-177) hands
+# over one fp32 2x2 rotation matrix per (position, pair) and ``apply_comfyui_rope`` (rope.py:180-212) applies it as
+#   x_out = freqs_cis[..., 0] * x_[..., 0];  x_out.addcmul_(freqs_cis[..., 1], x_[..., 1])
+# i.e. out[2i+e] = m[e][0] * x[2i] + m[e][1] * x[2i+1] in fp32.  torch evaluates the first product on its own and
+# fuses the second into the sum (one rounding for ``m[e][1] * x[2i+1] + first``); that is restated here with float64,
+# which holds the product of two fp32 values exactly (pinned against the two torch calls in tests/test_prep_oracle.py).
+# Positions past the table get the identity matrix (rope.py:133-148): unchanged rows.
+# ---------------------------------------------------------------------------------------------------------------
+def comfy_rope_matrices(ids: torch.Tensor, axes_dim=(44, 42, 42), theta: float = 10000.0) -> torch.Tensor:
+    """``EmbedND.forward`` without its broadcast dims: ``ids`` ``[L, n_axes]`` positions -> fp32 ``[L, sum(axes)/2, 2, 2]``
+    (``_comfy_rope``, rope.py:151-162: float64 frequencies, fp32 angles, ``[[cos, -sin], [sin, cos]]``)."""
+    parts = []
+    for a, dim in enumerate(axes_dim):
+        scale = torch.linspace(0, (dim - 2) / dim, steps=dim // 2, dtype=torch.float64)
+        omega = 1.0 / (theta**scale)
+        out = torch.einsum("...n,d->...nd", ids[..., a].to(torch.float32), omega)
+        out = torch.stack([torch.cos(out), -torch.sin(out), torch.sin(out), torch.cos(out)], dim=-1)
+        parts.append(out.reshape(*out.shape[:-1], 2, 2).to(torch.float32))
+    return torch.cat(parts, dim=-3)
+
+
+def comfy_rope_ref(x: torch.Tensor, matrices: torch.Tensor) -> torch.Tensor:
+    """``apply_comfyui_rope`` for one GPU: ``x`` ``[B, L, H, D]`` half, ``matrices`` fp32 ``[rows, D/2, 2, 2]``; rows of
+    ``x`` at or past ``rows`` stay as they are."""
+    B, L, H, D = x.shape
+    n = min(L, matrices.shape[0])
+    m = matrices[:n].to(torch.float32)[None, :, None]  # [1, n, 1, D/2, 2, 2]
+    xf = x[:, :n].float().reshape(B, n, H, D // 2, 2)
+    x0, x1 = xf[..., 0:1], xf[..., 1:2]  # [B, n, H, D/2, 1]
+    first = m[..., 0] * x0  # fp32 product, rounded
+    fused = (m[..., 1].double() * x1.double() + first.double()).float()  # exact product, one rounding of the sum
+    return torch.cat([fused.reshape(B, n, H, D).type_as(x), x[:, n:]], dim=1)
+
+
+def wan_comfy_prep_ref(x: torch.Tensor, weight, eps: float, matrices, num_heads: int) -> torch.Tensor:
+    """``[B, L, H*D]`` projection -> normed over the token row, viewed ``[B, L, H, D]``, rotated with the matrices."""
+    B, L, HD = x.shape
+    y = x if weight is None else rmsnorm_ref(x, weight, eps)
+    y = y.view(B, L, num_heads, HD // num_heads)
+    return y if matrices is None else comfy_rope_ref(y, matrices)

@@ -107,6 +107,50 @@ def test_prep_at_model_row_width_and_length(hip_device):
     _check_k(ws, pr.wan_prep_ref(kp, wk, 1e-6, grids, table, H), L)
 
 
+def _comfy_matrices(f, h, w):
+    ids = torch.zeros(f, h, w, 3)
+    ids[..., 0] += torch.arange(f).view(f, 1, 1)
+    ids[..., 1] += torch.arange(h).view(1, h, 1)
+    ids[..., 2] += torch.arange(w).view(1, 1, w)
+    return pr.comfy_rope_matrices(ids.reshape(-1, 3))
+
+
+@pytest.mark.parametrize(
+    "B,L,H,grid,dtype,norm",
+    [
+        (1, 24, 2, (2, 3, 4), torch.bfloat16, True),
+        (2, 300, 12, (3, 9, 11), torch.bfloat16, True),     # 297 rows rotate, 3 pass through (identity padding)
+        (1, 200, 40, (2, 10, 10), torch.bfloat16, True),    # the 14B row: 5120 channels
+        (1, 96, 4, (1, 8, 12), torch.float16, True),
+        (1, 96, 4, (4, 4, 6), torch.bfloat16, False),
+    ],
+)
+def test_quantizer_with_comfy_rope_is_bit_exact(hip_device, B, L, H, grid, dtype, norm):
+    """The Wan block with rope_func == "comfy" (wan_model.py:169-171, utils/rope.py:180-212): token-row RMSNorm, then
+    the 2x2-matrix rotation, on the way into the quantizer."""
+    print(f"case comfy B={B} L={L} H={H} grid={grid} {dtype} norm={norm}", flush=True)
+    qp, wq = _proj(B, L, H, seed=L + H + 7, dtype=dtype)
+    kp, wk = _proj(B, L, H, seed=L + H + 8, dtype=dtype)
+    m = _comfy_matrices(*grid)
+    # the module's layout, broadcast dims included (EmbedND.forward: [1, L_true, 1, D/2, 2, 2])
+    prep = WanPrep(q_norm_weight=wq if norm else None, k_norm_weight=wk if norm else None, eps=1e-6,
+                   comfy_freqs=m[None, :, None])
+    q4 = qp.view(B, L, H, 128).to(hip_device)
+    k4 = kp.view(B, L, H, 128).to(hip_device)
+    ws = sage_ops.workspace_for(q4, k4)
+    ws.blob.fill_(0x7F)
+    sage_ops.quant_q(q4, ws, 128**-0.5, prep=prep)
+    sage_ops.quant_k(k4, ws, prep=prep)
+    torch.cuda.synchronize()
+    assert sage_ops.quant_status(ws)[0] == 0
+    _check_q(ws, pr.wan_comfy_prep_ref(qp, wq if norm else None, 1e-6, m, H), 128**-0.5, L)
+    _check_k(ws, pr.wan_comfy_prep_ref(kp, wk if norm else None, 1e-6, m, H), L)
+    with pytest.raises(ValueError, match="either"):
+        WanPrep(comfy_freqs=m, freqs=pr.wan_rope_table(128), grid_sizes=[grid]).to_c(hip_device)
+    with pytest.raises(ValueError, match="comfy_freqs must be"):
+        WanPrep(comfy_freqs=m[:, :32]).to_c(hip_device)
+
+
 @pytest.mark.parametrize(
     "B,txt,img,H,dtype,norm,rope",
     [

@@ -232,3 +232,45 @@ def test_qwen_prep_composes_the_two_streams():
     assert torch.equal(out, torch.cat([txt, img], dim=1))
     assert torch.equal(pr.qwen_prep_ref(x, 10, None, None, 0.0, None, None), x)
     assert torch.equal(pr.qwen_prep_ref(x, 0, w_img, None, 1e-6, None, None), pr.head_rmsnorm_ref(x, w_img, 1e-6))
+
+
+# ----------------------------------------------------------------------------- the ComfyUI form of the Wan rotation (utils/rope.py:151-212)
+def _comfy_ids(f, h, w):
+    ids = torch.zeros(f, h, w, 3)
+    ids[..., 0] += torch.arange(f).view(f, 1, 1)
+    ids[..., 1] += torch.arange(h).view(1, h, 1)
+    ids[..., 2] += torch.arange(w).view(1, 1, w)
+    return ids.reshape(-1, 3)
+
+
+@pytest.mark.parametrize("L,dtype", [(1, torch.bfloat16), (37, torch.bfloat16), (64, torch.float16), (100, torch.bfloat16)])
+def test_comfy_rope_is_torchs_mul_then_addcmul(L, dtype):
+    g = torch.Generator().manual_seed(L)
+    x = (2.0 * torch.randn((2, L, 3, 128), generator=g)).to(dtype)
+    m = pr.comfy_rope_matrices(_comfy_ids(5, 4, 5)[:L] * 7.0)  # [L, 64, 2, 2]
+    # the reference's own two calls (rope.py:209-212) on its broadcast layout [1, L, 1, D/2, 2, 2]
+    freqs_cis = m[None, :, None]
+    x_ = x.to(dtype=freqs_cis.dtype).reshape(*x.shape[:-1], -1, 1, 2)
+    want = freqs_cis[..., 0] * x_[..., 0]
+    want.addcmul_(freqs_cis[..., 1], x_[..., 1])
+    want = want.reshape(*x.shape).type_as(x)
+    assert torch.equal(pr.comfy_rope_ref(x, m), want)
+
+
+def test_comfy_rope_agrees_with_the_default_rotation_and_pads_with_identity():
+    f, h, w = 3, 4, 5
+    n = f * h * w
+    x = _half((1, n + 6, 2, 128), 31)
+    m = pr.comfy_rope_matrices(_comfy_ids(f, h, w))
+    y = pr.comfy_rope_ref(x, m)
+    assert torch.equal(y[:, n:], x[:, n:])  # past the table: identity (rope.py:133-148)
+    # same angles as the complex128 table of the default path (44/42/42 channels per axis = 22/21/21 pairs), so
+    # the two rotations agree to fp32-angle accuracy, well inside a bf16 step for these small positions
+    ref = pr.rope_ref(x, [(f, h, w)], pr.wan_rope_table(128))
+    assert (y.float() - ref.float()).abs().max() <= 2.0**-7 * ref.float().abs().max()
+    assert (y != ref).float().mean() <= 0.02
+    # a rotation: pair norms survive; position (0, 0, 0) is the identity
+    n_in = x.double().reshape(1, n + 6, 2, 64, 2).norm(dim=-1)
+    n_out = y.double().reshape(1, n + 6, 2, 64, 2).norm(dim=-1)
+    assert ((n_in - n_out).abs() <= 2.0**-7 * n_in + 1e-6).all()
+    assert torch.equal(y[:, 0], x[:, 0])
