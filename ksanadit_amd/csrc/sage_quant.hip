@@ -47,6 +47,16 @@ __device__ __forceinline__ void load_row16(const uint16_t* row_ptr, bool valid, 
   widen8<DT>(b, out + 8);
 }
 
+// The same row as it sits in memory (two 16-byte loads), for code that wants the next row in flight while it works
+// on the current one.
+__device__ __forceinline__ void fetch_row16(const uint16_t* row_ptr, bool valid, uint4 (&raw)[2]) {
+  raw[0] = raw[1] = make_uint4(0, 0, 0, 0);
+  if (valid) {
+    raw[0] = *reinterpret_cast<const uint4*>(row_ptr);
+    raw[1] = *reinterpret_cast<const uint4*>(row_ptr + 8);
+  }
+}
+
 __device__ __forceinline__ float round_to_half_dtype(float x, int dtype) {
   if (dtype == KSANA_SAGE_BF16) return (float)(__bf16)x;
   return (float)(_Float16)x;
@@ -182,10 +192,12 @@ __device__ __forceinline__ void prep16_qwen(float* x, const PrepParams& pp, int 
   }
 }
 
-template <int DT>
+// KIND: PrepParams::kind, a template argument so that every kernel instantiation carries the registers of its own
+// variant only (with a run-time switch the three variants' table reads add up).
+template <int DT, int KIND>
 __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const RopeLds& rl, int b, int row, int h,
                                        int c16) {
-  if (pp.kind == 2) {  // uniform
+  if constexpr (KIND == 2) {
     prep16_qwen<DT>(x, pp, row, c16);
     return;
   }
@@ -201,7 +213,7 @@ __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const Rop
       x[4 * j + 3] = through_half<DT>((x[4 * j + 3] * r) * w.w);
     }
   }
-  if (pp.kind == 3) {  // uniform
+  if constexpr (KIND == 3) {
     // apply_comfyui_rope (utils/rope.py:180-212): out[2i+e] = m[e][0] * x[2i] + m[e][1] * x[2i+1] in fp32, the first
     // product rounded on its own, the second fused into the sum (what torch's mul followed by addcmul_ computes)
     if (pp.rot != nullptr && row < pp.rot_rows) {
@@ -251,10 +263,10 @@ __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const Rop
 // Dynamic LDS of the kernels that rotate: the staged factors.
 extern __shared__ __attribute__((aligned(16))) double2 s_rope_tables[];
 
-template <bool PRE>
+template <int PRE>
 __device__ __forceinline__ RopeLds maybe_stage_rope(const PrepParams& pp, int b, int row0, int nrows) {
   RopeLds rl{};
-  if constexpr (PRE) {
+  if constexpr (PRE == 1) {
     if (pp.freqs != nullptr && pp.lds_frames > 0) rl = stage_rope(pp, b, row0, nrows, s_rope_tables);
   }
   return rl;
@@ -292,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* _
 // OP 1: max |x| (order free).  OP 2: max |x - centre[d]| over the rows that exist (V smoothing: the
 // centre is the channel mean).  grid = (nch, H, B).
 // ---------------------------------------------------------------------------------------
-template <int DT, int OP, bool PRE>
+template <int DT, int OP, int PRE>
 __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
                                                                int64_t sH, int H, int L, float* __restrict__ part,
                                                                int nch, const PrepParams pp,
@@ -309,7 +321,7 @@ __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* _
     for (int i = 0; i < kMeanChunk / kSlots; ++i) {
       const int row = ch * kMeanChunk + i * kSlots + slot;
       load_row16<DT>(base + (int64_t)row * sL, row < L, rows[i]);
-      if (row < L) prep16<DT>(rows[i], pp, rl, b, row, h, c16);
+      if (row < L) prep16<DT, PRE>(rows[i], pp, rl, b, row, h, c16);
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = kSum ? rows[0][e] : fabsf(rows[0][e]);
@@ -540,7 +552,7 @@ __device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
 // workgroup handles 128 rows (4 per row slot).  grid = (lq_pad/128, H, B).  Output row-major
 // int8 [B, H, lq_pad, 128] and fp32 [B, H, lq_pad]; rows at or beyond L come out as zeros.
 // ---------------------------------------------------------------------------------------
-template <int DT, bool PRE>
+template <int DT, int PRE>
 __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __restrict__ q, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L, int lq_pad, float premul,
                                                            int8_t* __restrict__ q_i8, float* __restrict__ q_scale,
@@ -551,24 +563,13 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
   constexpr int kRowsPerWg = 128, R = kRowsPerWg / kSlots;
   const int64_t bh = (int64_t)b * H + h;
   const RopeLds rl = maybe_stage_rope<PRE>(pp, b, blk * kRowsPerWg, kRowsPerWg);
-  float x[R][16];
-#pragma unroll
-  for (int i = 0; i < R; ++i) {
-    const int row = blk * kRowsPerWg + i * kSlots + slot;
-    load_row16<DT>(base + (int64_t)row * sL, row < L, x[i]);
-    if constexpr (PRE) {
-      if (row < L) prep16<DT>(x[i], pp, rl, b, row, h, c16);
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < R; ++i) {
-    const int row = blk * kRowsPerWg + i * kSlots + slot;
-    fwht128(x[i], c16);
+  auto finish_row = [&](float* xr, int row) {
+    fwht128(xr, c16);
     float amax = 0.0f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      x[i][e] = x[i][e] * premul;
-      amax = fmaxf(amax, fabsf(x[i][e]));
+      xr[e] = xr[e] * premul;
+      amax = fmaxf(amax, fabsf(xr[e]));
     }
     amax = fmaxf(amax, lane_xor<1>(amax));
     amax = fmaxf(amax, lane_xor<2>(amax));
@@ -576,7 +577,34 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
     const bool nz = amax > 0.0f;
     const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
     if (c16 == 0) q_scale[bh * lq_pad + row] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
-    *reinterpret_cast<uint4*>(q_i8 + (bh * lq_pad + row) * kD + c16 * 16) = pack_int8x16(x[i], inv);
+    *reinterpret_cast<uint4*>(q_i8 + (bh * lq_pad + row) * kD + c16 * 16) = pack_int8x16(xr, inv);
+  };
+  if constexpr (PRE) {
+    // The norm and the rotation are arithmetic-heavy (vector fp64): one row at a time with only the next row's two
+    // loads in flight keeps the kernel at half the registers of "load all, then work", i.e. at twice the waves.
+    uint4 nxt[2];
+    fetch_row16(base + (int64_t)(blk * kRowsPerWg + slot) * sL, blk * kRowsPerWg + slot < L, nxt);
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int row = blk * kRowsPerWg + i * kSlots + slot;
+      const uint4 cur0 = nxt[0], cur1 = nxt[1];
+      if (i + 1 < R) fetch_row16(base + (int64_t)(row + kSlots) * sL, row + kSlots < L, nxt);
+      float xr[16];
+      widen8<DT>(cur0, xr);
+      widen8<DT>(cur1, xr + 8);
+      if (row < L) prep16<DT, PRE>(xr, pp, rl, b, row, h, c16);
+      finish_row(xr, row);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    float x[R][16];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int row = blk * kRowsPerWg + i * kSlots + slot;
+      load_row16<DT>(base + (int64_t)row * sL, row < L, x[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) finish_row(x[i], blk * kRowsPerWg + i * kSlots + slot);
   }
 }
 
@@ -586,7 +614,7 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
 // the attention kernel's int8 MFMA consumes it: fragment (t = row/32, s = 32-channel step)
 // is 64 lanes x 16 bytes, lane = 32*(16-channel half within the step) + row%32.
 // ---------------------------------------------------------------------------------------
-template <int DT, bool PRE>
+template <int DT, int PRE>
 __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L, int nkb,
                                                            const float* __restrict__ k_mean,
@@ -609,7 +637,7 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
     const bool valid = row < L;
     load_row16<DT>(base + (int64_t)row * sL, valid, x[i]);
     if constexpr (PRE) {
-      if (valid) prep16<DT>(x[i], pp, rl, b, row, h, c16);
+      if (valid) prep16<DT, PRE>(x[i], pp, rl, b, row, h, c16);
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -817,8 +845,11 @@ __device__ __forceinline__ void stage_partials(const float (&v)[kFinLoads], floa
   for (int j = 0; j < kFinLoads; ++j) s_part[(int)threadIdx.x + kThreads * j] = v[j];
 }
 
-template <int DT, bool PRE>
-__global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
+// With the Wan step folded in the kernel is asked to fit three waves per SIMD (168 registers; it spills ten of them):
+// a workgroup idles while it waits for its head's mean, and with two workgroups per compute unit instead of three
+// the kernel measured 23 % slower.
+template <int DT, int PRE>
+__global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
                                                                  int64_t sH, int H, int L, int nkb, int nch,
                                                                  float* __restrict__ part, float* k_mean, int dtype,
                                                                  int smooth, int8_t* __restrict__ k_tiles,
@@ -839,15 +870,22 @@ __global__ __launch_bounds__(kThreads) void quant_k_fused_kernel(const uint16_t*
   // ---- 1. the chunk, and its column sums in the specified order -------------------------------
   uint4 raw[kChunkRowsPerSlot][2];
   float acc[16];
+  uint4 nxt[2];
+  if constexpr (PRE) fetch_row16(base + (int64_t)(ch * kMeanChunk + slot) * sL, ch * kMeanChunk + slot < L, nxt);
 #pragma unroll
   for (int i = 0; i < kChunkRowsPerSlot; ++i) {
     const int row = ch * kMeanChunk + i * kSlots + slot;
     float x[16];
     if constexpr (PRE) {
-      load_row16<DT>(base + (int64_t)row * sL, row < L, x);
-      if (row < L) prep16<DT>(x, pp, rl, b, row, h, c16);
+      // one row at a time, the next row's loads in flight: see quant_q_kernel
+      const uint4 cur0 = nxt[0], cur1 = nxt[1];
+      if (i + 1 < kChunkRowsPerSlot) fetch_row16(base + (int64_t)(row + kSlots) * sL, row + kSlots < L, nxt);
+      widen8<DT>(cur0, x);
+      widen8<DT>(cur1, x + 8);
+      if (row < L) prep16<DT, PRE>(x, pp, rl, b, row, h, c16);
       raw[i][0] = narrow8<DT>(x);
       raw[i][1] = narrow8<DT>(x + 8);
+      __builtin_amdgcn_sched_barrier(0);
     } else {
       raw[i][0] = raw[i][1] = make_uint4(0, 0, 0, 0);
       if (row < L) {
@@ -1180,6 +1218,21 @@ __global__ void clear_ints_kernel(int* p, int n) {
     }                                            \
   } while (0)
 
+// KIND as a compile-time constant for the three variants of the folded step (PrepParams::kind)
+#define KSANA_DISPATCH_KIND(kind, ...)  \
+  do {                                  \
+    if ((kind) == 1) {                  \
+      constexpr int KIND = 1;           \
+      __VA_ARGS__;                      \
+    } else if ((kind) == 2) {           \
+      constexpr int KIND = 2;           \
+      __VA_ARGS__;                      \
+    } else {                            \
+      constexpr int KIND = 3;           \
+      __VA_ARGS__;                      \
+    }                                   \
+  } while (0)
+
 // Sizes the LDS copy of the rotation factors for kernels that give `rows_per_wg` consecutive rows to
 // a workgroup; returns the dynamic LDS bytes (0: the kernel reads the table directly).
 static size_t plan_rope_lds(PrepParams* pp, int B, int rows_per_wg) {
@@ -1211,15 +1264,16 @@ hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, fl
   const PrepParams none{};
   KSANA_DISPATCH_DT(x.dtype, {
     if (op == 2)
-      col_partial_kernel<DT, 2, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, centre);
+      col_partial_kernel<DT, 2, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, centre);
     else if (op == 1)
-      col_partial_kernel<DT, 1, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
+      col_partial_kernel<DT, 1, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
     else if (prep == nullptr)
-      col_partial_kernel<DT, 0, false><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
+      col_partial_kernel<DT, 0, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
-      col_partial_kernel<DT, 0, true><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, pp, nullptr);
+      KSANA_DISPATCH_KIND(pp.kind, (col_partial_kernel<DT, 0, KIND><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part,
+                                                                                        nch, pp, nullptr)));
     }
   });
   return hipGetLastError();
@@ -1243,13 +1297,13 @@ hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, fl
   const PrepParams none{};
   KSANA_DISPATCH_DT(q.dtype, {
     if (prep == nullptr)
-      quant_q_kernel<DT, false><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
+      quant_q_kernel<DT, 0><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
                                                         none);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, 128);
-      quant_q_kernel<DT, true><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
-                                                         pp);
+      KSANA_DISPATCH_KIND(pp.kind, (quant_q_kernel<DT, KIND><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad,
+                                                                                 premul, q_i8, q_scale, pp)));
     }
   });
   return hipGetLastError();
@@ -1261,13 +1315,13 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
   const PrepParams none{};
   KSANA_DISPATCH_DT(k.dtype, {
     if (prep == nullptr)
-      quant_k_kernel<DT, false><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
+      quant_k_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
                                                         none);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kBlkK);
-      quant_k_kernel<DT, true><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
-                                                         pp);
+      KSANA_DISPATCH_KIND(pp.kind, (quant_k_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb,
+                                                                                 k_mean, k_tiles, k_scale, pp)));
     }
   });
   return hipGetLastError();
@@ -1322,20 +1376,23 @@ hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb,
   hipError_t e = hipSuccess;
   KSANA_DISPATCH_DT(k.dtype, {
     if (prep == nullptr) {
-      const int resident = resident_workgroups(quant_k_fused_kernel<DT, false>, 0);
+      const int resident = resident_workgroups(quant_k_fused_kernel<DT, 0>, 0);
       if (2 * nch <= resident) {
-        quant_k_fused_kernel<DT, false><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
+        quant_k_fused_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
                                                                 k.dtype, smooth, k_tiles, k_scale, none, sy);
         *used = true;
       }
     } else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
-      if (2 * nch <= resident_workgroups(quant_k_fused_kernel<DT, true>, lds)) {
-        quant_k_fused_kernel<DT, true><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
-                                                                 k.dtype, smooth, k_tiles, k_scale, pp, sy);
-        *used = true;
-      }
+      KSANA_DISPATCH_KIND(pp.kind, {
+        // lds != 0 only for kind 1; the cached answer (lds == 0) is kept per instantiation
+        if (2 * nch <= resident_workgroups(quant_k_fused_kernel<DT, KIND>, lds)) {
+          quant_k_fused_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
+                                                                   k.dtype, smooth, k_tiles, k_scale, pp, sy);
+          *used = true;
+        }
+      });
     }
   });
   if (*used) e = hipGetLastError();
