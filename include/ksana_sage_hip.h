@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 14
+#define KSANA_SAGE_ABI_VERSION 15
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -67,7 +67,10 @@ typedef struct ksana_sage_shape {
   int32_t Hkv; /* key/value heads; Hq % Hkv == 0                            */
   int32_t Lq;  /* query sequence length                                     */
   int32_t Lk;  /* key/value sequence length                                 */
-  int32_t D;   /* head size (128)                                           */
+  int32_t D;   /* head size: 128, or 64.  Rows of 64 channels are treated as    */
+               /* rows of 128 whose upper half is zero (same workspace size,    */
+               /* same kernels; o rows are 64 channels).  The folded norm /     */
+               /* rotation step (ksana_sage_*_prep) needs 128.                  */
 } ksana_sage_shape;
 
 /* Byte offsets of the sub-buffers inside the workspace blob (each 256-byte aligned). */

@@ -35,7 +35,7 @@ from ..config import KsanaAttentionBackend, KsanaAttentionConfig
 from ..sage_ops import sageattn
 from .base import KsanaAttentionBackendImpl
 
-SUPPORTED_HEAD_SIZES = (128,)
+SUPPORTED_HEAD_SIZES = (64, 128)  # 64 runs zero-padded to 128 channels inside the library
 
 
 class SageAttentionImpl(KsanaAttentionBackendImpl):

@@ -167,7 +167,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   if (p.k_lens != nullptr) lk = min(max(p.k_lens[b], 0), p.Lk);  // uniform: a scalar load
   auto write_zero_rows = [&]() {  // softmax over no key: the output rows are defined as zeros
     const int q = q0 + l32;
-    if (q < p.Lq) {
+    if (q < p.Lq && 64 * hh < p.d_out) {
       uint4* orow = reinterpret_cast<uint4*>(p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH + 64 * hh);
 #pragma unroll
       for (int i = 0; i < 8; ++i) orow[i] = make_uint4(0, 0, 0, 0);
@@ -673,7 +673,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   for (int i = 0; i < 8; ++i) {
     const int idx = i * 64 + lane, r = idx >> 4, c = idx & 15;  // row r of the wave, 16-byte piece c of it
     const uint4 piece = *reinterpret_cast<const uint4*>(stage + r * kPitch + 16 * c);
-    if (q0 + r < p.Lq) *reinterpret_cast<uint4*>(obase + (int64_t)(q0 + r) * p.o.sL + 8 * c) = piece;
+    if (q0 + r < p.Lq && 8 * c < p.d_out) *reinterpret_cast<uint4*>(obase + (int64_t)(q0 + r) * p.o.sL + 8 * c) = piece;
   }
 }
 
@@ -688,7 +688,7 @@ __global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p
   const int bhk = b * p.Hkv + h / (p.Hq / p.Hkv);
   const int row = blockIdx.y * 8 + (threadIdx.x >> 5), d = (threadIdx.x & 31) * 4;
   const int q = qwg * kAttnQPerWg + row;
-  if (q >= p.Lq) return;
+  if (q >= p.Lq || d >= p.d_out) return;
   uint16_t* orow = p.o.ptr + b * p.o.sB + (int64_t)q * p.o.sL + h * p.o.sH;
   if (p.q_lens != nullptr && q >= min(max(p.q_lens[b], 0), p.Lq)) {  // a row that does not take part: zeros
     *reinterpret_cast<uint2*>(orow + d) = make_uint2(0, 0);

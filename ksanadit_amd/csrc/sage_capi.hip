@@ -42,7 +42,8 @@ int check_shape(const ksana_sage_shape* s) {
     return fail(KSANA_SAGE_EINVAL, "shape has a non-positive extent (B=%d Hq=%d Hkv=%d Lq=%d Lk=%d)", s->B, s->Hq,
                 s->Hkv, s->Lq, s->Lk);
   if (s->Hq % s->Hkv != 0) return fail(KSANA_SAGE_EINVAL, "Hq=%d is not a multiple of Hkv=%d", s->Hq, s->Hkv);
-  if (s->D != ksana_sage::kD) return fail(KSANA_SAGE_ENOTSUP, "head size %d not supported (only 128)", s->D);
+  if (s->D != ksana_sage::kD && s->D != 64)
+    return fail(KSANA_SAGE_ENOTSUP, "head size %d not supported (128, or 64 run zero-padded to 128)", s->D);
   if (s->Lk > 262144) return fail(KSANA_SAGE_ENOTSUP, "Lk=%d exceeds 262144 (K scales of one head are kept in LDS)", s->Lk);
   if ((int64_t)s->B * s->Hq > 65535 * 8 || s->Hq > 65535 || s->B > 65535)
     return fail(KSANA_SAGE_EINVAL, "B*H too large for the launch grid");
@@ -74,8 +75,8 @@ int hip_fail(hipError_t e, const char* what) {
   return fail(KSANA_SAGE_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-ksana_sage::InTensor in_tensor(const void* p, int dtype, const int64_t st[4]) {
-  return ksana_sage::InTensor{static_cast<const uint16_t*>(p), st[0], st[1], st[2], dtype};
+ksana_sage::InTensor in_tensor(const void* p, int dtype, const int64_t st[4], int D = ksana_sage::kD) {
+  return ksana_sage::InTensor{static_cast<const uint16_t*>(p), st[0], st[1], st[2], dtype, D};
 }
 
 template <typename T>
@@ -162,9 +163,10 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
 // Validates `prep` for one tensor (`weight` is that tensor's norm weight) and fills the kernel-side
 // parameters.  *out stays nullptr when there is nothing to apply.
 int make_prep(const ksana_sage_prep* prep, const float* weight, const char* name, const int64_t st[4], int B, int L,
-              float* inv_rms, ksana_sage::PrepParams* pp, const ksana_sage::PrepParams** out) {
+              int D, float* inv_rms, ksana_sage::PrepParams* pp, const ksana_sage::PrepParams** out) {
   *out = nullptr;
   if (!prep) return 0;
+  if (D != ksana_sage::kD) return fail(KSANA_SAGE_ENOTSUP, "the folded norm / rotation step needs head size 128, got %d", D);
   if (prep->kind != KSANA_SAGE_PREP_WAN && prep->kind != KSANA_SAGE_PREP_WAN_COMFY && prep->kind != KSANA_SAGE_PREP_QWEN)
     return fail(KSANA_SAGE_EINVAL, "prep kind %d unknown", prep->kind);
   if (prep->kind == KSANA_SAGE_PREP_QWEN) {
@@ -299,7 +301,7 @@ int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t st[4], const
   ksana_sage_workspace_layout(s, &l);
   ksana_sage::PrepParams pp;
   const ksana_sage::PrepParams* ppp = nullptr;
-  if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", st, s->B, s->Lq, ws_at<float>(ws, l.q_rms),
+  if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", st, s->B, s->Lq, s->D, ws_at<float>(ws, l.q_rms),
                          &pp, &ppp))
     return rc;
   if (ppp && ppp->inv_rms) {
@@ -310,7 +312,7 @@ int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t st[4], const
   // one fp32 product, then an exact power of two (1/128 undoes the unnormalised Hadamard
   // transforms of Q and K): part of the quantizer specification
   const float premul = (sm_scale * 1.4426950408889634f) * 0.0078125f;
-  hipError_t e = ksana_sage::launch_quant_q(in_tensor(q, dtype, st), s->B, s->Hq, s->Lq, l.lq_pad, premul,
+  hipError_t e = ksana_sage::launch_quant_q(in_tensor(q, dtype, st, s->D), s->B, s->Hq, s->Lq, l.lq_pad, premul,
                                             ws_at<int8_t>(ws, l.q_i8), ws_at<float>(ws, l.q_scale),
                                             static_cast<hipStream_t>(stream), ppp);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_q launch");
@@ -331,13 +333,13 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
   ksana_sage_ws_layout l;
   ksana_sage_workspace_layout(s, &l);
   hipStream_t hs = static_cast<hipStream_t>(stream);
-  const ksana_sage::InTensor kt = in_tensor(k, dtype, st);
+  const ksana_sage::InTensor kt = in_tensor(k, dtype, st, s->D);
   const int bhk = s->B * s->Hkv;
   if (part == nullptr) part = ws_at<float>(ws, l.k_part);
   if (sync_words == nullptr) sync_words = ws_at<int>(ws, l.k_sync);
   ksana_sage::PrepParams pp;
   const ksana_sage::PrepParams* ppp = nullptr;
-  if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", st, s->B, s->Lk, ws_at<float>(ws, l.k_rms),
+  if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", st, s->B, s->Lk, s->D, ws_at<float>(ws, l.k_rms),
                          &pp, &ppp))
     return rc;
   hipError_t e = hipSuccess;
@@ -407,7 +409,7 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], con
   ksana_sage_ws_layout l;
   ksana_sage_workspace_layout(s, &l);
   hipStream_t hs = static_cast<hipStream_t>(stream);
-  const ksana_sage::InTensor vt = in_tensor(v, dtype, st);
+  const ksana_sage::InTensor vt = in_tensor(v, dtype, st, s->D);
   const int bhk = s->B * s->Hkv;
   float* v_mean = ws_at<float>(ws, l.v_mean);
   hipError_t e = hipSuccess;
@@ -532,6 +534,7 @@ int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[
   p.mask_sB = block_mask ? mask_st[0] : 0;
   p.mask_sH = block_mask ? mask_st[1] : 0;
   p.causal = causal ? 1 : 0;
+  p.d_out = s->D;
   hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
 }
@@ -584,9 +587,9 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
     ksana_sage::PrepParams pp;
     const ksana_sage::PrepParams* ppp = nullptr;
     float dummy = 0.0f;  // only the validation matters here
-    if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", q_st, s->B, s->Lq, &dummy, &pp, &ppp))
+    if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", q_st, s->B, s->Lq, s->D, &dummy, &pp, &ppp))
       return rc;
-    if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", k_st, s->B, s->Lk, &dummy, &pp, &ppp))
+    if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", k_st, s->B, s->Lk, s->D, &dummy, &pp, &ppp))
       return rc;
   }
   if (int rc = ksana_sage_quant_q_prep(q, dtype, q_st, s, prep, sm_scale, ws, stream)) return rc;

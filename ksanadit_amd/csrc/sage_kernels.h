@@ -20,6 +20,7 @@ struct InTensor {
   const uint16_t* ptr;
   int64_t sB, sL, sH;  // element strides of [B, L, H, D]; D stride is 1
   int dtype;           // KSANA_SAGE_BF16 / KSANA_SAGE_FP16
+  int D = 128;         // channels per row that exist: 128, or 64 (the kernels then read the upper 64 as zeros)
 };
 
 struct OutTensor {
@@ -129,6 +130,7 @@ struct AttnParams {
   float* split_ml;
   int split_first_wg, n_split;  // filled in by the launcher
   int wg_waves;  // 0: the launcher picks the workgroup shape; 4 or 8: forced (for measurements and tests)
+  int d_out;     // channels of an output row that exist: 128, or 64 (head size 64 runs zero-padded to 128)
 };
 constexpr int kMaxSplitPartials = 256;  // (workgroups beyond the last full round) x (runs each) never exceeds this
 constexpr int kMinTilesPerSplit = 8;    // a run shorter than this does not repay its prologue

@@ -306,12 +306,13 @@ __global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* _
 // ---------------------------------------------------------------------------------------
 template <int DT, int OP, int PRE>
 __global__ __launch_bounds__(kThreads) void col_partial_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
-                                                               int64_t sH, int H, int L, float* __restrict__ part,
+                                                               int64_t sH, int H, int L_all, int d_in, float* __restrict__ part,
                                                                int nch, const PrepParams pp,
                                                                const float* __restrict__ centre) {
   constexpr bool kSum = OP == 0;
   const int ch = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const uint16_t* base = x + b * sB + h * sH + c16 * 16;
   const RopeLds rl = maybe_stage_rope<PRE>(pp, b, ch * kMeanChunk, kMeanChunk);
   float acc[16];
@@ -554,11 +555,12 @@ __device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
 // ---------------------------------------------------------------------------------------
 template <int DT, int PRE>
 __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __restrict__ q, int64_t sB, int64_t sL,
-                                                           int64_t sH, int H, int L, int lq_pad, float premul,
+                                                           int64_t sH, int H, int L_all, int d_in, int lq_pad, float premul,
                                                            int8_t* __restrict__ q_i8, float* __restrict__ q_scale,
                                                            const PrepParams pp) {
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const uint16_t* base = q + b * sB + h * sH + c16 * 16;
   constexpr int kRowsPerWg = 128, R = kRowsPerWg / kSlots;
   const int64_t bh = (int64_t)b * H + h;
@@ -616,12 +618,13 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
 // ---------------------------------------------------------------------------------------
 template <int DT, int PRE>
 __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
-                                                           int64_t sH, int H, int L, int nkb,
+                                                           int64_t sH, int H, int L_all, int d_in, int nkb,
                                                            const float* __restrict__ k_mean,
                                                            int8_t* __restrict__ k_tiles, float* __restrict__ k_scale,
                                                            const PrepParams pp) {
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const int64_t bh = (int64_t)b * H + h;
   const uint16_t* base = k + b * sB + h * sH + c16 * 16;
   float km[16];
@@ -669,12 +672,13 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
 // ---------------------------------------------------------------------------------------
 template <int DT, bool CENTRE>
 __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __restrict__ v, int64_t sB, int64_t sL,
-                                                           int64_t sH, int H, int L, int nkb,
+                                                           int64_t sH, int H, int L_all, int d_in, int nkb,
                                                            const float* __restrict__ v_inv,
                                                            const float* __restrict__ v_mean,
                                                            uint8_t* __restrict__ v_tiles) {
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const int64_t bh = (int64_t)b * H + h;
   const uint16_t* base = v + b * sB + h * sH + c16 * 16;
   constexpr int kStride = kD + 16;  // LDS row pitch in bytes
@@ -850,7 +854,7 @@ __device__ __forceinline__ void stage_partials(const float (&v)[kFinLoads], floa
 // the kernel measured 23 % slower.
 template <int DT, int PRE>
 __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
-                                                                 int64_t sH, int H, int L, int nkb, int nch,
+                                                                 int64_t sH, int H, int L_all, int d_in, int nkb, int nch,
                                                                  float* __restrict__ part, float* k_mean, int dtype,
                                                                  int smooth, int8_t* __restrict__ k_tiles,
                                                                  float* __restrict__ k_scale, const PrepParams pp,
@@ -858,6 +862,7 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
   const int bh = blockIdx.x / nch, ch = blockIdx.x - bh * nch;
   const int b = bh / H, h = bh - b * H;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const int wave = t >> 6, lane = t & 63;
   const uint16_t* base = k + b * sB + h * sH + c16 * 16;
   const RopeLds rl = maybe_stage_rope<PRE>(pp, b, ch * kMeanChunk, kMeanChunk);
@@ -950,7 +955,7 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
       }
     }
     if (t < kD) {
-      const float mean = round_to_half_dtype(__fdiv_rn(tot, (float)L), dtype);
+      const float mean = round_to_half_dtype(__fdiv_rn(tot, (float)L_all), dtype);
       s_mean[t] = mean;
       publish_f32(k_mean + bh * kD + t, mean);
       complete_accesses();
@@ -1005,13 +1010,14 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
 // order of quant_v_kernel.
 template <int DT>
 __global__ __launch_bounds__(kThreads) void quant_v_fused_kernel(const uint16_t* __restrict__ v, int64_t sB, int64_t sL,
-                                                                 int64_t sH, int H, int L, int nkb, int nch,
+                                                                 int64_t sH, int H, int L_all, int d_in, int nkb, int nch,
                                                                  float* __restrict__ part, float* v_scale, float* v_inv,
                                                                  float* __restrict__ v_mean,
                                                                  uint8_t* __restrict__ v_tiles, const HeadSync sy) {
   const int bh = blockIdx.x / nch, ch = blockIdx.x - bh * nch;
   const int b = bh / H, h = bh - b * H;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const int wave = t >> 6, lane = t & 63;
   const uint16_t* base = v + b * sB + h * sH + c16 * 16;
   __shared__ float s_w[4][kD];
@@ -1264,15 +1270,15 @@ hipError_t launch_col_partial(const InTensor& x, int B, int H, int L, int op, fl
   const PrepParams none{};
   KSANA_DISPATCH_DT(x.dtype, {
     if (op == 2)
-      col_partial_kernel<DT, 2, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, centre);
+      col_partial_kernel<DT, 2, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, x.D, part, nch, none, centre);
     else if (op == 1)
-      col_partial_kernel<DT, 1, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
+      col_partial_kernel<DT, 1, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, x.D, part, nch, none, nullptr);
     else if (prep == nullptr)
-      col_partial_kernel<DT, 0, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part, nch, none, nullptr);
+      col_partial_kernel<DT, 0, 0><<<grid, block, 0, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, x.D, part, nch, none, nullptr);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
-      KSANA_DISPATCH_KIND(pp.kind, (col_partial_kernel<DT, 0, KIND><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, part,
+      KSANA_DISPATCH_KIND(pp.kind, (col_partial_kernel<DT, 0, KIND><<<grid, block, lds, s>>>(x.ptr, x.sB, x.sL, x.sH, H, L, x.D, part,
                                                                                         nch, pp, nullptr)));
     }
   });
@@ -1297,12 +1303,12 @@ hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, fl
   const PrepParams none{};
   KSANA_DISPATCH_DT(q.dtype, {
     if (prep == nullptr)
-      quant_q_kernel<DT, 0><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, q_i8, q_scale,
+      quant_q_kernel<DT, 0><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, q.D, lq_pad, premul, q_i8, q_scale,
                                                         none);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, 128);
-      KSANA_DISPATCH_KIND(pp.kind, (quant_q_kernel<DT, KIND><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad,
+      KSANA_DISPATCH_KIND(pp.kind, (quant_q_kernel<DT, KIND><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, q.D, lq_pad,
                                                                                  premul, q_i8, q_scale, pp)));
     }
   });
@@ -1315,12 +1321,12 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
   const PrepParams none{};
   KSANA_DISPATCH_DT(k.dtype, {
     if (prep == nullptr)
-      quant_k_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, k_mean, k_tiles, k_scale,
+      quant_k_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb, k_mean, k_tiles, k_scale,
                                                         none);
     else {
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kBlkK);
-      KSANA_DISPATCH_KIND(pp.kind, (quant_k_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb,
+      KSANA_DISPATCH_KIND(pp.kind, (quant_k_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb,
                                                                                  k_mean, k_tiles, k_scale, pp)));
     }
   });
@@ -1378,7 +1384,7 @@ hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb,
     if (prep == nullptr) {
       const int resident = resident_workgroups(quant_k_fused_kernel<DT, 0>, 0);
       if (2 * nch <= resident) {
-        quant_k_fused_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
+        quant_k_fused_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb, nch, part, k_mean,
                                                                 k.dtype, smooth, k_tiles, k_scale, none, sy);
         *used = true;
       }
@@ -1388,7 +1394,7 @@ hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb,
       KSANA_DISPATCH_KIND(pp.kind, {
         // lds != 0 only for kind 1; the cached answer (lds == 0) is kept per instantiation
         if (2 * nch <= resident_workgroups(quant_k_fused_kernel<DT, KIND>, lds)) {
-          quant_k_fused_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, nkb, nch, part, k_mean,
+          quant_k_fused_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb, nch, part, k_mean,
                                                                    k.dtype, smooth, k_tiles, k_scale, pp, sy);
           *used = true;
         }
@@ -1410,7 +1416,7 @@ hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb,
   KSANA_DISPATCH_DT(v.dtype, {
     const int resident = resident_workgroups(quant_v_fused_kernel<DT>, 0);
     if (2 * nch <= resident) {
-      quant_v_fused_kernel<DT><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, nch, part, v_scale, v_inv,
+      quant_v_fused_kernel<DT><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, v.D, nkb, nch, part, v_scale, v_inv,
                                                        v_mean, v_tiles, sy);
       *used = true;
     }
@@ -1424,9 +1430,9 @@ hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const
   const dim3 grid(nkb, H, B), block(kThreads);
   KSANA_DISPATCH_DT(v.dtype, {
     if (v_mean != nullptr)
-      quant_v_kernel<DT, true><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, v_inv, v_mean, v_tiles);
+      quant_v_kernel<DT, true><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, v.D, nkb, v_inv, v_mean, v_tiles);
     else
-      quant_v_kernel<DT, false><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, nkb, v_inv, nullptr, v_tiles);
+      quant_v_kernel<DT, false><<<grid, block, 0, s>>>(v.ptr, v.sB, v.sL, v.sH, H, L, v.D, nkb, v_inv, nullptr, v_tiles);
   });
   return hipGetLastError();
 }

@@ -106,7 +106,7 @@ class SageWorkspace:
     @property
     def q_i8(self):
         s, l = self.shape, self.layout
-        return self._view(l.q_i8, s.B * s.Hq * l.lq_pad * s.D, torch.int8, (s.B, s.Hq, l.lq_pad, s.D))
+        return self._view(l.q_i8, s.B * s.Hq * l.lq_pad * PAD_D, torch.int8, (s.B, s.Hq, l.lq_pad, PAD_D))
 
     @property
     def q_scale(self):
@@ -126,7 +126,7 @@ class SageWorkspace:
     @property
     def k_mean(self):
         s, l = self.shape, self.layout
-        return self._view(l.k_mean, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
+        return self._view(l.k_mean, s.B * s.Hkv * PAD_D * 4, torch.float32, (s.B, s.Hkv, PAD_D))
 
     @property
     def v_tiles(self):
@@ -136,14 +136,14 @@ class SageWorkspace:
     @property
     def v_scale(self):
         s, l = self.shape, self.layout
-        return self._view(l.v_scale, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
+        return self._view(l.v_scale, s.B * s.Hkv * PAD_D * 4, torch.float32, (s.B, s.Hkv, PAD_D))
 
 
     @property
     def v_mean(self):
         """Channel means the V quantizer took off (zeros unless it ran with ``smooth_v``)."""
         s, l = self.shape, self.layout
-        return self._view(l.v_mean, s.B * s.Hkv * s.D * 4, torch.float32, (s.B, s.Hkv, s.D))
+        return self._view(l.v_mean, s.B * s.Hkv * PAD_D * 4, torch.float32, (s.B, s.Hkv, PAD_D))
 
     @property
     def q_rms(self):
@@ -376,6 +376,7 @@ def _k_lens_arg(k_lens, batch: int, device: torch.device, name: str = "k_lens"):
     return k_lens.to(device=device, dtype=torch.int32).contiguous()
 
 
+PAD_D = 128  # channels per row of the quantized operands: head size 64 runs zero-padded to 128
 MASK_BLKQ, MASK_BLKK = 128, 64  # query rows / keys per block-mask entry
 
 

@@ -60,6 +60,16 @@ def _to_bhld_f32(x: torch.Tensor) -> torch.Tensor:
     return x.permute(0, 2, 1, 3).to(torch.float32).contiguous()
 
 
+def pad_head_dim(x: torch.Tensor, to: int = 128) -> torch.Tensor:
+    """Head size 64 (rule 7 of the specification): every row of Q, K and V is extended to 128 channels with zeros and
+    rules 1-6 apply to the extended rows unchanged.  The transform of an extended row is the 64-point transform of the
+    row twice in a row, so ``(H q') . (H k') = 128 q . k`` as for head size 128; the extended channels of V quantize to
+    zero with scale zero, and the output keeps the first 64 channels."""
+    d = x.shape[-1]
+    assert d <= to
+    return x if d == to else torch.nn.functional.pad(x, (0, to - d))
+
+
 def q_premul(sm_scale: float, D: int = 128) -> torch.Tensor:
     """``c`` of rule 4, as a 0-d fp32 tensor (``2**-7`` is ``1/D`` for the head size 128)."""
     c = torch.tensor(sm_scale, dtype=torch.float32) * torch.tensor(LOG2E, dtype=torch.float32)

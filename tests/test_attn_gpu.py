@@ -114,7 +114,7 @@ def test_op_contract_on_gpu(hip_device):
     with pytest.raises(ValueError):
         attn(q[0], k[0], v[0])
     with pytest.raises(NotImplementedError):
-        sage_ops.sageattn(torch.zeros(1, 8, 1, 64, device=hip_device, dtype=torch.bfloat16), *(torch.zeros(1, 8, 1, 64, device=hip_device, dtype=torch.bfloat16),) * 2)
+        sage_ops.sageattn(torch.zeros(1, 8, 1, 96, device=hip_device, dtype=torch.bfloat16), *(torch.zeros(1, 8, 1, 96, device=hip_device, dtype=torch.bfloat16),) * 2)
     with pytest.raises(RuntimeError):
         sage_ops.sageattn(*(torch.zeros(1, 8, 1, 128, dtype=torch.bfloat16),) * 3)
 
@@ -646,6 +646,62 @@ SCHEME_BUDGET = {
 # Full shapes, all heads, per group of 8 heads against torch SDPA on the GPU: worst element over 8 x L x 128 outputs
 # relative to that group's max|O| (the tail of the same int8 effect over 8 - 40 times more rows than above)
 FULL_SIZE_WORST = {"wan14b_480p": 0.20, "wan14b_720p": 0.22, "qwen_cfg": 0.15}
+
+
+@pytest.mark.parametrize("B,Lq,Lk,Hq,Hkv,causal", [(2, 300, 300, 4, 4, False), (1, 257, 1100, 4, 2, False), (1, 500, 500, 2, 2, True)])
+def test_head_size_64(hip_device, B, Lq, Lk, Hq, Hkv, causal):
+    """Head size 64 through the operator (the selector now keeps the Sage backend for it): against SDPA, against the
+    emulation on the quantized (zero-extended) operands, with per-batch key counts and a strided output slot."""
+    print(f"case D=64 B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv} causal={causal}", flush=True)
+    g = torch.Generator().manual_seed(Lq * 3 + Lk)
+    q = torch.randn((B, Lq, Hq, 64), generator=g).to(torch.bfloat16)
+    k = (torch.randn((B, Lk, Hkv, 64), generator=g) + 1.5 * torch.randn((1, 1, Hkv, 64), generator=g)).to(torch.bfloat16)
+    v = torch.randn((B, Lk, Hkv, 64), generator=g).to(torch.bfloat16)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    op = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN))(num_heads=Hq, head_size=64, causal=causal, num_kv_heads=Hkv)
+    out = op(qd, kd, vd)
+    assert op.backend_type == KsanaAttentionBackend.SAGE_ATTN
+    assert out.shape == q.shape and out.dtype == q.dtype and out.is_contiguous()
+    rep = Hq // Hkv
+    ref = sdpa_ref(q, k.repeat_interleave(rep, dim=2), v.repeat_interleave(rep, dim=2), causal=causal)
+    assert _cos(out.cpu(), ref) >= COS_MIN
+    # short sequences of unit-variance data: |O| ~ 0.1-1 and the scheme's own error scales with it (as in
+    # test_attention_vs_oracles_small); the reference's absolute bounds are checked in the next test
+    err = (out.cpu().float() - ref.float()).abs()
+    assert err.max() <= 0.08 * ref.float().abs().max() and err.mean() <= 0.01 * ref.float().abs().max()
+    ws = sage_ops.workspace_for(qd, kd)
+    ws.blob.fill_(0x7F)
+    o2 = sage_ops.sageattn(qd, kd, vd, workspace=ws, is_causal=causal)
+    assert torch.equal(o2, out)
+    emul = _emul_from_ws(ws, Lq, Lk, q.dtype, causal=causal)  # [B, Lq, Hq, 128]; the upper 64 channels are zeros
+    assert torch.count_nonzero(emul[..., 64:]) == 0
+    assert (o2.cpu().float() - emul[..., :64].float()).abs().max() <= 2e-2 * emul.float().abs().max().item()
+    if not causal:
+        k_lens = torch.tensor([Lk - 37] + [Lk // 2] * (B - 1), dtype=torch.int32)
+        o3 = sage_ops.sageattn(qd, kd, vd, k_lens=k_lens.to(hip_device)).cpu()
+        for b in range(B):
+            n = int(k_lens[b])
+            rb = sdpa_ref(q[b : b + 1], k[b : b + 1, :n].repeat_interleave(rep, dim=2), v[b : b + 1, :n].repeat_interleave(rep, dim=2))
+            assert _cos(o3[b : b + 1], rb) >= COS_MIN
+        # both workgroup shapes write the 128-byte rows of a head-size-64 output and nothing beyond them
+        slab = torch.full((B, Lq, Hq, 128), 7.0, dtype=q.dtype, device=hip_device)
+        for waves in (4, 8):
+            sage_ops.attn_fwd(ws, slab[..., :64], wg_waves=waves)
+            same_shape = sage_ops.attn_fwd(ws, torch.empty_like(o2), wg_waves=waves)  # (a cut into key runs differs by shape)
+            assert torch.equal(slab[..., :64], same_shape) and bool((slab[..., 64:] == 7.0).all())
+            assert _cos(same_shape.cpu(), ref) >= COS_MIN
+
+
+def test_reference_sage_check_at_head_size_64(hip_device):
+    """The reference's own Sage check (tests/ksana/attention_op_test.py:157-186: fp16 randn, max < 1e-1, mean < 1e-2)
+    with its shape's head size halved."""
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn((2, 32, 64, 64), generator=g).to(torch.float16).to(hip_device) for _ in range(3))
+    op = pick_attn_op(KsanaAttentionConfig(backend=KsanaAttentionBackend.SAGE_ATTN))(num_heads=64, head_size=64, causal=False)
+    out = op(q, k, v)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+    diff = (out - ref).abs()
+    assert diff.max().item() < 1e-1 and diff.mean().item() < 1e-2
 
 
 def test_wan_cross_attention_at_model_size(hip_device):

@@ -55,7 +55,7 @@ def test_workspace_layout_headline_shape():
 
 @pytest.mark.parametrize(
     "args,exc",
-    [((1, 4, 4, 16, 16, 64), NotImplementedError), ((1, 4, 3, 16, 16, 128), ValueError), ((1, 4, 4, 0, 16, 128), ValueError),
+    [((1, 4, 4, 16, 16, 96), NotImplementedError), ((1, 4, 3, 16, 16, 128), ValueError), ((1, 4, 4, 0, 16, 128), ValueError),
      ((0, 4, 4, 16, 16, 128), ValueError), ((1, 4, 4, 16, 262145, 128), NotImplementedError), ((1, 70000, 70000, 16, 16, 128), ValueError),
      ((1, 4, 4, (1 << 24) + 1, 16, 128), NotImplementedError), ((8, 65535, 65535, 1 << 20, 16, 128), NotImplementedError)],
 )
@@ -113,6 +113,13 @@ def test_entry_points_validate_before_touching_the_gpu():
     odd = _capi.Strides(64 * 2 * 128, 2 * 128 + 4, 128, 1)
     assert lib.ksana_sage_quant_q(fake, _capi.BF16, odd, C.byref(shape), 0.1, fake, null) == _capi.EINVAL
     assert lib.ksana_sage_quant_q(fake, _capi.BF16, st, C.byref(shape), 0.1, null, null) == _capi.EINVAL  # workspace
+    lay = _capi.WsLayout()
+    assert lib.ksana_sage_workspace_layout(C.byref(_capi.Shape(1, 2, 2, 64, 64, 64)), C.byref(lay)) == 0  # head size 64
+    lay128 = _capi.WsLayout()
+    assert lib.ksana_sage_workspace_layout(C.byref(shape), C.byref(lay128)) == 0
+    assert lay.total_bytes == lay128.total_bytes  # it runs zero-padded to 128 channels
+    assert lib.ksana_sage_workspace_layout(C.byref(_capi.Shape(1, 2, 2, 64, 64, 96)), C.byref(lay)) == _capi.ENOTSUP
+    assert b"head size 96" in lib.ksana_sage_last_error()
     long_k = _capi.Shape(1, 2, 2, 64, 131073, 128)  # causal masking keeps its tile list in LDS: Lk <= 131072
     assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(long_k), null, 1, 0, null) == _capi.ENOTSUP
     assert b"causal" in lib.ksana_sage_last_error()

@@ -567,3 +567,26 @@ def test_sage_emul_survives_outliers():
     q, k, v = make_inputs("wan14b_480p", heads=1, seq=2048)
     ref, out = sdpa_ref(q, k, v), sage_emul_ref(q, k, v)
     assert _cos(out, ref) >= 0.999
+
+
+def test_head_size_64_rows_extended_with_zeros_keep_the_products():
+    """Rule 7: a 64-channel row extended with zeros transforms into the 64-point transform written twice, so the
+    product of two transformed rows is still 128 times the product of the rows (exact on small integers), the extended
+    K mean is zero there and the extended V channels quantize to zero codes with scale zero."""
+    g = torch.Generator().manual_seed(64)
+    q = torch.randint(-8, 9, (1, 5, 2, 64), generator=g).to(torch.bfloat16)
+    k = torch.randint(-8, 9, (1, 7, 2, 64), generator=g).to(torch.bfloat16)
+    qp, kp = qr.pad_head_dim(q), qr.pad_head_dim(k)
+    assert qp.shape[-1] == 128 and torch.equal(qp[..., :64], q) and torch.count_nonzero(qp[..., 64:]) == 0
+    hq, hk = qr.fwht_ref(qp.float()), qr.fwht_ref(kp.float())
+    h64 = qr.fwht_ref(q.float())
+    assert torch.equal(hq, torch.cat([h64, h64], dim=-1))
+    exact = torch.einsum("blhd,bmhd->bhlm", q.double(), k.double())
+    got = torch.einsum("blhd,bmhd->bhlm", hq.double(), hk.double())
+    assert torch.equal(got, 128.0 * exact)
+    _, _, km = qr.quant_k_ref(kp)
+    assert torch.count_nonzero(km[..., 64:]) == 0
+    v = torch.randn((1, 7, 2, 64), generator=g).to(torch.bfloat16)
+    v8, vs = qr.quant_v_ref(qr.pad_head_dim(v))
+    assert torch.count_nonzero(v8.view(torch.uint8)[..., 64:]) == 0 and torch.count_nonzero(vs[..., 64:]) == 0
+    assert torch.equal(qr.pad_head_dim(qp), qp)

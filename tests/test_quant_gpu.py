@@ -51,6 +51,24 @@ def _check_against_oracle(q, k, v, dev, sm_scale=None, smooth_k=True):
         assert torch.count_nonzero(full[:, :, Lk:]) == 0, "v padding rows not zero"
 
 
+@pytest.mark.parametrize("B,Lq,Lk,Hq,Hkv,dtype", [(1, 70, 70, 2, 2, torch.bfloat16), (2, 300, 520, 4, 2, torch.float16)])
+def test_quantizer_bit_exact_head_size_64(hip_device, B, Lq, Lk, Hq, Hkv, dtype):
+    """Head size 64: the kernels read the upper 64 channels as zeros; the oracle quantizes the zero-extended tensors."""
+    print(f"case D=64 B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(Lq + Lk)
+    q = torch.randn((B, Lq, Hq, 64), generator=g).to(dtype)
+    k = (torch.randn((B, Lk, Hkv, 64), generator=g) + 2.0 * torch.randn((1, 1, Hkv, 64), generator=g)).to(dtype)
+    v = (1.5 * torch.randn((B, Lk, Hkv, 64), generator=g)).to(dtype)
+    ws = _run_quant(q, k, v, hip_device, 64**-0.5, True)
+    qi, qs = qr.quant_q_ref(qr.pad_head_dim(q), 64**-0.5)
+    ki, ks, km = qr.quant_k_ref(qr.pad_head_dim(k))
+    v8, vs = qr.quant_v_ref(qr.pad_head_dim(v))
+    assert torch.equal(ws.q_i8.cpu()[:, :, :Lq], qi) and torch.equal(ws.q_scale.cpu()[:, :, :Lq], qs)
+    assert torch.equal(ws.k_mean.cpu(), km.float()) and torch.equal(ws.k_scale.cpu(), ks)
+    assert torch.equal(untile_k(ws.k_tiles.cpu(), Lk), ki)
+    assert torch.equal(ws.v_scale.cpu(), vs) and torch.equal(untile_v(ws.v_tiles.cpu(), Lk), v8.view(torch.uint8))
+
+
 def _rand_qkv(B, Lq, Lk, Hq, Hkv, seed, dtype=torch.bfloat16):
     g = torch.Generator().manual_seed(seed)
     q = torch.randn((B, Lq, Hq, 128), generator=g)
