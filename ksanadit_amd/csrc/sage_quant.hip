@@ -526,21 +526,17 @@ __device__ __forceinline__ float block_max(float v, float* s_red) {
   return fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
 }
 
-// clamp(rne(x * inv), -127, 127) as int8, sixteen at a time.  The product is rounded to fp32 first (the
-// specification's order), clamped (clamping before or after the rounding to an integer gives the same integer), and
-// then rounded to an integer by adding 1.5 * 2^23: at that magnitude the fp32 grid is the integers and the addition
-// rounds to nearest, ties to even, so the low byte of the sum is the two's-complement int8.  Three instructions per
-// value plus three byte-gathers per four, instead of round / clamp / convert / mask / shift / or.
+// rne(x * inv) as int8, sixteen at a time, the product exact: one fused multiply-add onto 1.5 * 2^23, where the fp32
+// grid is the integers, rounds the exact sum to nearest, ties to even, and leaves the two's-complement int8 in the low
+// byte.  No clamp: |x| <= amax and inv = fl(127 / amax) keep |x * inv| below 127.5.  One instruction per value plus
+// three byte-gathers per four.
 __device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
   uint32_t w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     uint32_t z[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float y = __builtin_amdgcn_fmed3f(x[4 * i + j] * inv, -127.0f, 127.0f);
-      z[j] = __float_as_uint(y + 12582912.0f);
-    }
+    for (int j = 0; j < 4; ++j) z[j] = __float_as_uint(__fmaf_rn(x[4 * i + j], inv, 12582912.0f));
     const uint32_t lo = __builtin_amdgcn_perm(z[1], z[0], 0x0c0c0400u);  // bytes 0, 1 <- low bytes of z0, z1
     const uint32_t hi = __builtin_amdgcn_perm(z[3], z[2], 0x04000c0cu);  // bytes 2, 3 <- low bytes of z2, z3
     w[i] = lo | hi;

@@ -30,8 +30,9 @@ call sites leave open is frozen HERE, and the HIP kernels reproduce it bit for b
    product and an exact power-of-two scaling), so the attention kernel exponentiates with
    ``exp2`` directly.
 5. int8: ``amax = max|x|`` over a block, ``scale = amax / 127``, ``inv = 127 / amax`` (IEEE
-   divisions; both 0 when ``amax == 0``), ``x_i8 = clamp(rne(x * inv), -127, 127)`` with
-   ``rne`` = round-half-to-even (``torch.round``).  A K block is ``BLKK`` = 64 key rows
+   divisions; both 0 when ``amax == 0``), ``x_i8 = rne(x * inv)`` with the product EXACT (not first rounded to
+   fp32: what a fused multiply-add onto ``1.5 * 2**23`` leaves in its low byte) and ``rne`` = round-half-to-even;
+   ``|x * inv| <= 127 (1 + 2**-24)`` by construction, so no clamp is needed (one is kept here as a guard).  A K block is ``BLKK`` = 64 key rows
    (sage_sla.py:204; a ragged last block uses its valid rows only).  A Q block is ONE query
    row (``BLKQ`` = 1): per-token scales cost nothing in the attention kernel, where a lane
    owns one query column, and keep a Q outlier from degrading 127 other rows.
@@ -133,7 +134,8 @@ def _block_int8(x: torch.Tensor, blk: int):
     qmax = torch.full_like(amax, 127.0)
     scale = torch.where(nz, amax / qmax, torch.zeros_like(amax))
     inv = torch.where(nz, qmax / safe, torch.zeros_like(amax))
-    y = torch.round(xb * inv.unsqueeze(-1)).clamp_(-127.0, 127.0)
+    # float64 holds the product of two fp32 values exactly (48 significant bits); torch.round is half-to-even
+    y = torch.round(xb.double() * inv.unsqueeze(-1).double()).clamp_(-127.0, 127.0)
     xi = y.to(torch.int8).view(B, H, nb * blk, D)[:, :, :L].contiguous()
     return xi, scale
 

@@ -5,6 +5,8 @@ fp8 format definition, and invariants the mathematics fixes."""
 
 import math
 
+from fractions import Fraction
+
 import numpy as np
 import pytest
 import torch
@@ -93,7 +95,7 @@ def test_k_mean_close_to_f64_and_constant_columns():
 
 # ------------------------------------------------------------------ int8 block quantizer
 def _scalar_block_int8(x2d, blk):
-    """Independent scalar implementation of rule 4 on a [L, D] float32 numpy array."""
+    """Independent scalar implementation of rule 5 on a [L, D] float32 numpy array."""
     L, D = x2d.shape
     nb = (L + blk - 1) // blk
     out = np.zeros((L, D), dtype=np.int8)
@@ -112,9 +114,10 @@ def _scalar_block_int8(x2d, blk):
         inv = f32(f32(127.0) / amax)
         for r in rows:
             for d in range(D):
-                y = f32(x2d[r, d] * inv)
-                n = float(np.rint(y))  # rint = half to even
-                out[r, d] = int(max(-127.0, min(127.0, n)))
+                # the exact product (rationals), rounded once, half to even (Python's round of a Fraction)
+                n = round(Fraction(float(x2d[r, d])) * Fraction(float(inv)))
+                assert -127 <= n <= 127  # |x| <= amax and inv = fl(127 / amax): never beyond 127 (1 + 2^-24)
+                out[r, d] = n
     return out, scales
 
 
@@ -211,8 +214,8 @@ def test_quant_hand_computed_blocks():
     xi, xs, _ = qr.quant_k_ref(x, smooth_k=False)
     # row 3 = (1,-20,1,1) -> (-17, 21, -21, 21); other rows -> (4,0,0,0); block amax 21
     inv = f32(f32(127.0) / f32(21.0))
-    assert xi[0, 0, 3].tolist() == [int(np.rint(f32(v) * inv)) for v in (-17, 21, -21, 21)]
-    assert xi[0, 0, 0].tolist() == [int(np.rint(f32(4.0) * inv)), 0, 0, 0]
+    assert xi[0, 0, 3].tolist() == [round(Fraction(v) * Fraction(float(inv))) for v in (-17, 21, -21, 21)]
+    assert xi[0, 0, 0].tolist() == [round(Fraction(4) * Fraction(float(inv))), 0, 0, 0]
     assert xs[0, 0].tolist() == [float(f32(21.0) / f32(127.0)), float(f32(4.0) / f32(127.0))]
     # ragged tail: last block's scale comes from its valid rows only
     x = torch.ones((1, 70, 1, D), dtype=torch.bfloat16)
