@@ -276,18 +276,34 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
       const bool two = kMaskRows == 2 && 2 * qwg + 1 < nqm;
       const int wg_tiles = p.causal ? min(nkb, ((qwg * kRowsWg + kRowsWg - 1) >> 6) + 1) : nkb;
       int base = 0;
-      for (int j0 = 0; j0 < wg_tiles; j0 += 64) {
-        const int j = j0 + lane;
-        int f0 = 0, f1 = 0;
-        if (j < wg_tiles) {
-          f0 = !masked || m0[j] != 0;
-          f1 = two && (!masked || m0[p.nkb + j] != 0);
+      // eight chunks of 64 tiles at a time: their mask bytes are requested together, so a list of 512 tiles costs
+      // one memory latency instead of eight
+      for (int jb = 0; jb < wg_tiles; jb += 512) {
+        int8_t b0[8], b1[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const int j = jb + 64 * c + lane;
+          b0[c] = b1[c] = 1;
+          if (masked && j < wg_tiles) {
+            b0[c] = m0[j];
+            if (two) b1[c] = m0[p.nkb + j];
+          }
         }
-        const bool keep = (f0 | f1) != 0;
-        const unsigned long long bal = __ballot(keep);
-        const int pre = __builtin_amdgcn_mbcnt_hi((unsigned)(bal >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)bal, 0));
-        if (keep) s_list[base + pre] = j | (f0 << 16) | (f1 << 17);
-        base += __popcll(bal);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const int j = jb + 64 * c + lane;
+          if (jb + 64 * c >= wg_tiles) break;  // uniform
+          int f0 = 0, f1 = 0;
+          if (j < wg_tiles) {
+            f0 = b0[c] != 0;
+            f1 = two && b1[c] != 0;
+          }
+          const bool keep = (f0 | f1) != 0;
+          const unsigned long long bal = __ballot(keep);
+          const int pre = __builtin_amdgcn_mbcnt_hi((unsigned)(bal >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)bal, 0));
+          if (keep) s_list[base + pre] = j | (f0 << 16) | (f1 << 17);
+          base += __popcll(bal);
+        }
       }
       if (lane == 0) s_list[kListMax] = base;
     }
@@ -302,6 +318,26 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
   }
   if (tid < 2 * kD) s_vs[tid] = tid < kD ? p.v_scale[(int64_t)bhk * kD + tid] : p.v_mean[(int64_t)bhk * kD + tid - kD];
+  // Causal calls: the list is in key order, so the entries this wave takes part in (tile <= the one on its diagonal)
+  // are the first n_mine, and the diagonal tile, if listed, is the last of them.  Both are found once here; the key
+  // loop then compares loop positions instead of looking list entries up.
+  int n_mine = n_tiles, jdiag = -1;  // wave-uniform
+  if constexpr (kSparse) {
+    if (p.causal) {
+      if (p.block_mask == nullptr) {  // the list is 0, 1, 2, ...
+        n_mine = min(n_tiles, my_last + 1);
+      } else {
+        int cnt = 0;
+        for (int j0 = 0; j0 < n_tiles; j0 += 64) {
+          const int jx = j0 + lane;
+          const bool le = jx < n_tiles && (s_list[jx] & 0xffff) <= my_last;
+          cnt += __popcll(__ballot(le));
+        }
+        n_mine = cnt;
+      }
+      if (n_mine > 0 && (__builtin_amdgcn_readfirstlane(s_list[n_mine - 1]) & 0xffff) == my_last) jdiag = n_mine - 1;
+    }
+  }
   // key tile behind loop position jj, and whether this wave's mask row asks for it
   auto tile_of = [&](int jj) -> int {
     if constexpr (kSparse) return __builtin_amdgcn_readfirstlane(s_list[jj]) & 0xffff;
@@ -309,14 +345,15 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   };
   auto mine_at = [&](int jj) -> bool {
     if constexpr (kSparse) {
+      if constexpr (kW == 4) return jj < n_mine;  // one mask row per workgroup: every listed tile is wanted
       const int e = __builtin_amdgcn_readfirstlane(s_list[jj]);
-      return ((e >> (16 + (kW == 8 ? (wave >> 2) : 0))) & 1) != 0 && (e & 0xffff) <= my_last;
+      return ((e >> (16 + (wave >> 2))) & 1) != 0 && jj < n_mine;
     }
     return true;
   };
   // causal only: list position jj holds the tile on this wave's diagonal
   auto diag_at = [&](int jj) -> bool {
-    if constexpr (kSparse) return p.causal && tile_of(jj) == my_last;
+    if constexpr (kSparse) return jj == jdiag;
     return false;
   };
   // scores of keys beyond the row's own position drop below every real score ...
@@ -563,9 +600,10 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     mx_cur = max(max(pm[0], pm[1]), max(pm[2], pm[3]));
     ks_cur = ks_nxt;
     if constexpr (kSparse) {
-      const int keep = mine ? -1 : 0;
+      if (!mine) {  // wave-uniform and rare: a tile this wave's row does not take part in contributes nothing
 #pragma unroll
-      for (int i = 0; i < 8; ++i) pf[i] &= keep;
+        for (int i = 0; i < 8; ++i) pf[i] = 0;
+      }
       if (diag_at(j)) causal_probs(pf);
     }
     // after this barrier: tile j+2 is visible to every wave, and nobody reads tile j-1 any more
