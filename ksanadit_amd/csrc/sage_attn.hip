@@ -47,6 +47,16 @@ struct WgShape {
   static constexpr int kAhead = kW == 8 ? 4 : 2;       // global -> LDS copies are issued this many tiles ahead
   static constexpr int kCopies = 2 * (8 / kW);         // 1 KiB copy instructions per wave and tile (K and V^T halves)
   static constexpr int kRingBytes = kStages * 2 * kTileBytes;
+  // The 4-wave shape keeps K tiles and V^T tiles in two rings of kStages slots each (same memory).  A K tile is
+  // read one step BEFORE the step of its probabilities and its V^T tile one step AFTER, so in one ring of whole
+  // tiles two K halves are always dead; in its own ring K can be requested kStages tiles ahead instead of two.
+  // That matters where tiles miss the L2 (block masks): with two tiles ahead and every copy awaited at the end of the
+  // step it was issued in, a copy has one step (about a microsecond) to arrive; now it has three.
+  static constexpr bool kTwoRings = kW == 4;
+  static constexpr int kAheadK = kTwoRings ? kStages : kAhead;
+  // copies that may still be in flight at the barrier that ends a step: those of the newest (kAhead - 2) tiles in
+  // one ring; with two rings everything issued in this step and the one before
+  static constexpr int kInFlight = kTwoRings ? 2 * kCopies : kCopies * (kAhead - 2);
 };
 constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f
 constexpr float kMagicF = 12582912.0f;
@@ -391,41 +401,64 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // keys >= lk live only in the last key tile, which (if the list holds it) is the last entry
   const bool has_tail = (lk & (kBlkK - 1)) != 0 && tile_of(n_tiles - 1) == nkb - 1;
   const int n_main = has_tail ? n_tiles - 1 : n_tiles;  // entries handled by the pipelined loop
-  auto issue_copy = [&](int tile) {
-    // clamped: past the end the last tile is copied again into a stage nobody reads any more,
-    // which keeps the loop free of branches and the outstanding-copy count constant
+  // LDS slot of a tile's K half / V^T half
+  auto k_slot = [&](int tile) -> uint8_t* {
+    if constexpr (Shape::kTwoRings) return smem + (tile & (kStages - 1)) * kTileBytes;
+    return smem + (tile & (kStages - 1)) * kStageBytes;
+  };
+  auto v_slot = [&](int tile) -> uint8_t* {
+    if constexpr (Shape::kTwoRings) return smem + (kStages + (tile & (kStages - 1))) * kTileBytes;
+    return smem + (tile & (kStages - 1)) * kStageBytes + kTileBytes;
+  };
+  // clamped: past the end the last tile is copied again into a slot nobody reads any more,
+  // which keeps the loop free of branches and the outstanding-copy count constant
+  auto copy_half = [&](const uint8_t* src, int tile, uint8_t* dst) {
     const int jl = tile_of(min(tile, n_tiles - 1));
-    const uint8_t* dst = smem + (tile & (kStages - 1)) * kStageBytes;
 #pragma unroll
-    for (int c = 0; c < 8 / kW; ++c) {  // this wave's 1 KiB slices of the two tiles: slice c * kW + wave
+    for (int c = 0; c < 8 / kW; ++c) {  // this wave's 1 KiB slices of the tile: slice c * kW + wave
       const int slice = c * kW + wave;
-      const unsigned off = (unsigned)(slice * 64 + lane) * 16;
-      lds_copy16(k_src + (int64_t)jl * kTileBytes, off, dst + slice * 1024);
-      lds_copy16(v_src + (int64_t)jl * kTileBytes, off, dst + slice * 1024 + kTileBytes);
+      lds_copy16(src + (int64_t)jl * kTileBytes, (unsigned)(slice * 64 + lane) * 16, dst + slice * 1024);
     }
   };
-  // wait until every copy except those of the newest (kAhead - 2) tiles has landed, then meet
-  // the other waves.  Plain s_barrier: a fence here would drain ALL copies and undo the prefetch.
+  // the copies of loop step j (step -1: nothing; the prologue below brings the first tiles in)
+  auto issue_copy = [&](int j) {
+    copy_half(v_src, j + kAhead, v_slot(j + kAhead));  // first: it is awaited first
+    copy_half(k_src, j + Shape::kAheadK, k_slot(j + Shape::kAheadK));
+  };
+  // wait until every copy except the newest Shape::kInFlight has landed, then meet the other waves.
+  // Plain s_barrier: a fence here would drain ALL copies and undo the prefetch.
   auto tile_barrier = [&]() {
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Shape::kCopies * (kAhead - 2)) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Shape::kInFlight) : "memory");
   };
 
   // Every ordinary global load above (Q fragments, scales) must have returned before the first
   // asynchronous copy is issued: the compiler would otherwise drain ALL memory operations,
   // copies included, at the first use of a loaded value inside the loop.
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  // The last stage's V half is read (times P = 0) by the first loop iteration: make it finite.
+  // The V^T slot of "tile -1" is read (times P = 0) by the first loop iteration: make it finite.
 #pragma unroll
   for (int c = 0; c < 8 / kW; ++c)
-    *reinterpret_cast<uint4*>(smem + (kStages - 1) * kStageBytes + kTileBytes + (c * kThreadsAttn + tid) * 16) = make_uint4(0, 0, 0, 0);
+    *reinterpret_cast<uint4*>(v_slot(-1) + (c * kThreadsAttn + tid) * 16) = make_uint4(0, 0, 0, 0);
+  if constexpr (Shape::kTwoRings) {
 #pragma unroll
-  for (int t = 0; t < kAhead; ++t) issue_copy(t);
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(Shape::kCopies * (kAhead - 2)) : "memory");  // tiles 0, 1 visible
+    for (int t = 0; t < kAhead; ++t) copy_half(v_src, t, v_slot(t));
+#pragma unroll
+    for (int t = 0; t < Shape::kAheadK; ++t) copy_half(k_src, t, k_slot(t));
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  } else {
+#pragma unroll
+    for (int t = 0; t < kAhead; ++t) {  // tile by tile: the oldest copies are the ones awaited
+      copy_half(k_src, t, k_slot(t));
+      copy_half(v_src, t, v_slot(t));
+    }
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(Shape::kInFlight) : "memory");  // tiles 0, 1 visible
+  }
 
   if (!active) {
     // same copy / barrier sequence as the active waves
+    if constexpr (Shape::kTwoRings) __builtin_amdgcn_s_barrier();
     for (int j = 0; j < n_main; ++j) {
-      issue_copy(j + kAhead);
+      issue_copy(j);
       tile_barrier();
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -498,7 +531,9 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   };
 
   v16i s_a[2], s_b[2];
-  qk_tile(smem, lane, qf, magic, s_a);
+  qk_tile(k_slot(0), lane, qf, magic, s_a);
+  // two rings: step 0 requests K tile kStages into the slot of K tile 0, which every wave must have read by then
+  if constexpr (Shape::kTwoRings) __builtin_amdgcn_s_barrier();
   if (diag_at(0)) causal_scores(s_a);
   int mx_cur = lane_max(s_a);  // this lane's maximum of the tile whose probabilities come next
   float ks_cur = s_ks[0];
@@ -516,8 +551,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   v8i pf_x = {0, 0, 0, 0, 0, 0, 0, 0}, pf_y = {0, 0, 0, 0, 0, 0, 0, 0};
   float alpha_prev = 1.0f;
   auto tile_step = [&](int j, v16i (&s_cur)[2], v16i (&s_nxt)[2], const v8i& pf_prev, v8i& pf) {
-    const uint8_t* kst = smem + ((j + 1) & (kStages - 1)) * kStageBytes;
-    const uint8_t* vst = smem + ((j - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
+    const uint8_t* kst = k_slot(j + 1);
+    const uint8_t* vst = v_slot(j - 1);
     auto k_frag = [&](int i) { return *reinterpret_cast<const v4i*>(kst + (((i & 1) * 4 + (i >> 1)) * 64 + lane) * 16); };
     auto v_frag = [&](int dt) {
       const v4i lo = *reinterpret_cast<const v4i*>(vst + ((dt * 2 + 0) * 64 + lane) * 16);
@@ -533,7 +568,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     kf[2] = k_frag(2);
     const float ks_nxt = s_ks[min(j + 1, n_tiles - 1)];
     const bool mine = mine_at(j);
-    issue_copy(j + kAhead);
+    issue_copy(j);
     if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
     // row sums of tile j-1: 64 matrix cycles that run under the max finalisation below
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
@@ -619,9 +654,14 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     if (j < n_main) tile_step(j, s_a, s_b, pf_x, pf_y);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may outlive the workgroup's LDS
+  if constexpr (Shape::kTwoRings) {
+    // the peeled last tile's V^T half was requested two steps ago; the loop's last barrier vouches only for copies
+    // three steps old, so the waves meet once more after each has seen its own copies land (uniform condition)
+    if (has_tail) __builtin_amdgcn_s_barrier();
+  }
   if (n_main > 0) {  // drain: PV of the last pipelined tile
     scale_o(alpha_prev);
-    const uint8_t* vst = smem + ((n_main - 1) & (kStages - 1)) * kStageBytes + kTileBytes;
+    const uint8_t* vst = v_slot(n_main - 1);
     const v8i pf_last = (n_main & 1) ? pf_y : pf_x;  // written by the last step
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_last);
@@ -659,7 +699,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
         pf[4 * t + g] = w & (int)keep;
       }
     if (diag_at(jj)) causal_probs(pf);
-    const uint8_t* vst = smem + (jj & (kStages - 1)) * kStageBytes + kTileBytes;
+    const uint8_t* vst = v_slot(jj);
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf);
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, lacc, 0, 0, 0, 0, 0, 0);
