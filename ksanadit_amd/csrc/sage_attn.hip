@@ -60,7 +60,16 @@ struct WgShape {
 };
 constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f
 constexpr float kMagicF = 12582912.0f;
-constexpr float kPShift = 8.0f;           // P is scaled by 2^8 before the e4m3 cast
+// P is scaled by 2^6 before the e4m3 cast, and the reference point of a row (its "running maximum") is moved only when
+// a tile's maximum exceeds it by more than kLazyMax octaves: probabilities then reach 2^(6 + 2.7) = 416 < 448, the
+// largest e4m3 value, and the accumulators are rescaled in a few per cent of the steps instead of up to half of them
+// (rows of flat attention set a new maximum every few tiles, by small amounts).  An e4m3 rounding does not depend on
+// the power of two in front, so the result differs only where probabilities fall off the subnormal end, 2^-15 of the
+// reference point.
+// The piecewise-linear path keeps 2^8 and moves the reference point at every new maximum: its code formula is wrong
+// for the subnormal codes (it fades them linearly), which must stay 2^-14 below the true maximum to be harmless.
+constexpr float kPShift = 6.0f, kPShiftPwl = 8.0f;
+constexpr float kLazyMax = 2.7f, kLazyMaxPwl = 0.0f;
 constexpr int kStageBytes = 2 * kTileBytes;  // K tile + V tile
 constexpr int kSparseMaxKeyTiles4 = 1024;    // 4-wave workgroups keep a shorter tile list so that two fit a compute unit
 constexpr int kMaxKeyTiles = 4096;           // K scales of one head are kept in LDS: Lk <= 262144
@@ -494,8 +503,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     }
     // the accumulator read as fp32 is magic + dot, so one fma gives sc * dot (mneg = -magic * sc)
     const float m_tile = __builtin_fmaf(__int_as_float(imax), sc, mneg);
-    const float m_new = fmaxf(m_run, m_tile);
-    const float alpha = fast_exp2(m_run - m_new);
+    const float m_new = m_tile > m_run + (kPwlExp ? kLazyMaxPwl : kLazyMax) ? m_tile : m_run;  // -inf at the first tile: always taken
+    const float alpha = fast_exp2(m_run - m_new);                     // exactly 1 where the reference point stays
     m_run = m_new;
     return alpha;
   };
@@ -506,8 +515,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   //   exact:  p = exp2(x) on the transcendental unit, then the hardware e4m3 conversion;
   //   kPwlExp: the e4m3 CODE is computed directly, code = rne(8*x + 55.5) (saturating at 0): an
   //           e4m3 code is a 3-bit-mantissa logarithm, so this is exp2 with a piecewise-linear
-  //           mantissa - two VALU slots per key instead of 3.5, no transcendental.  x <= 8 keeps
-  //           the code <= 120, clear of the NaN code 127.
+  //           mantissa - two VALU slots per key instead of 3.5, no transcendental.  x <= 8.7 keeps
+  //           the code <= 125, clear of the NaN code 127.
   auto pack4 = [&](int s0, int s1, int s2, int s3, float sc, float c) -> int {
     if constexpr (kPwlExp) {
       // here sc and c arrive pre-multiplied by 8, c with the +55.5 folded in
@@ -579,7 +588,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     alpha_prev = mine ? update_max(mx_cur, sc, mneg) : 1.0f;
     // exponent of key r: x = sc*dot - m_run + shift, with the magic folded into the constant
     // (which is therefore off by at most ~1.5 integer steps of the dot product)
-    const float c = (kPShift - m_run) + mneg;
+    const float c = ((kPwlExp ? kPShiftPwl : kPShift) - m_run) + mneg;
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     int pm[4];
@@ -680,7 +689,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     const float sc = qs * s_ks[jj];
     const float mneg = -kMagicF * sc;
     scale_o(update_max(lane_max(s_cur), sc, mneg));
-    const float c = (kPShift - m_run) + mneg;
+    const float c = ((kPwlExp ? kPShiftPwl : kPShift) - m_run) + mneg;
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     v8i pf;

@@ -5,7 +5,7 @@ The attention output of the path is compared with the reference's torch SDPA bac
 and on the same seeded inputs, into the contributions of the three quantizations, switched on one after the other:
 
     A   INT8 Q and K (Hadamard-transformed, per-row / per-64-key scales), exact softmax, exact V
-    B   A + the probabilities rounded to e4m3 (relative to the row maximum, scaled by 2^8)
+    B   A + the probabilities rounded to e4m3 (relative to the row maximum, scaled by 2^P_SHIFT)
     C   B + V rounded to per-channel e4m3, result rounded to bf16        = the scheme the kernel implements
 
 each against float64 attention on the bf16 inputs.  ``python -m oracle.error_budget <workload> [heads]`` prints the

@@ -24,8 +24,15 @@ import torch
 from .quant_ref import BLKK, BLKQ, FP8_MAX, e4m3fn_decode_table, quant_k_ref, quant_q_ref, quant_v_ref
 
 # P is scaled by 2**P_SHIFT before the fp8 cast so that small probabilities stay above the
-# e4m3 subnormal floor (2**-9); the factor cancels in O = (P V) / rowsum(P).
-P_SHIFT = 8.0
+# e4m3 subnormal floor (2**-9); the factor cancels in O = (P V) / rowsum(P).  The online form moves a row's reference
+# point (its "running maximum") only when a tile's maximum exceeds it by more than LAZY_MAX octaves, as the kernel
+# does: probabilities then reach 2**(P_SHIFT + LAZY_MAX) = 416 < 448.
+P_SHIFT = 6.0
+LAZY_MAX = 2.7
+# The piecewise-linear path keeps 2**8 and follows every new maximum: its code formula fades the subnormal codes
+# linearly, which is harmless only far below the true maximum.
+P_SHIFT_PWL = 8.0
+LAZY_MAX_PWL = 0.0
 
 
 def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
@@ -129,9 +136,10 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                     # a key the row may not see scores magic - 2**22, below every real dot product
                     xt_max = xt if allow is None else torch.where(allow, xt, torch.tensor(magic - 4194304.0))
                     m_tile = (xt_max.amax(dim=1, keepdim=True).double() * sc.double() + mneg.double()).float()  # fma
-                    m_new = torch.maximum(m, m_tile)
-                    alpha = torch.exp2(m - m_new)
-                    c = (P_SHIFT - m_new) + mneg
+                    lazy = torch.tensor(LAZY_MAX if exact_exp2 else LAZY_MAX_PWL, dtype=torch.float32)
+                    m_new = torch.where(m_tile > m + lazy, m_tile, m)
+                    alpha = torch.exp2(m - m_new)  # 1 where the reference point stays, 0 at a row's first tile
+                    c = ((P_SHIFT if exact_exp2 else P_SHIFT_PWL) - m_new) + mneg
                     if exact_exp2:
                         e = (xt.double() * sc.double() + c.double()).float()
                         p8 = torch.exp2(e).clamp(max=FP8_MAX).to(torch.float8_e4m3fn).float()
@@ -171,7 +179,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 o = torch.where(l > 0, o, torch.zeros_like(o))
             else:
                 m = s.amax(dim=1, keepdim=True)
-                p8 = p_to_e4m3(s - m + P_SHIFT, exact_exp2)
+                p8 = p_to_e4m3(s - m + (P_SHIFT if exact_exp2 else P_SHIFT_PWL), exact_exp2)
                 l = p8.sum(dim=1, keepdim=True)
                 o = (p8 @ vf) * v_scale[b, hk][None, :] / l
                 if v_mean is not None:
