@@ -287,9 +287,13 @@ def workspace_for(q: torch.Tensor, k: torch.Tensor) -> SageWorkspace:
 
 
 def _check_qwen_rows(prep, L: int) -> None:
-    """The image table of a ``QwenPrep`` must cover the rows behind the text rows."""
-    if isinstance(prep, QwenPrep) and prep.img_freqs is not None and prep.img_freqs.shape[0] < L - prep.txt_len:
+    """The tables of a ``QwenPrep`` must cover their segments: the kernels index them by row without a bound."""
+    if not isinstance(prep, QwenPrep):
+        return
+    if prep.img_freqs is not None and prep.img_freqs.shape[0] < L - prep.txt_len:
         raise ValueError(f"img_freqs has {prep.img_freqs.shape[0]} rows, the image segment {L - prep.txt_len}")
+    if prep.txt_freqs is not None and prep.txt_freqs.shape[0] < min(prep.txt_len, L):
+        raise ValueError(f"txt_freqs has {prep.txt_freqs.shape[0]} rows, the text segment {min(prep.txt_len, L)}")
 
 
 def quant_q(q: torch.Tensor, ws: SageWorkspace, sm_scale: float, prep: "WanPrep | QwenPrep | None" = None) -> None:
@@ -491,23 +495,22 @@ def sageattn(
     sm_scale = D**-0.5 if sm_scale is None else float(sm_scale)
     ws = workspace_for(q, k) if workspace is None else workspace
     ws.require(q.device, B=B, Hq=Hq, Hkv=k.shape[2], Lq=Lq, Lk=k.shape[1], D=D)
-    out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lib = _capi.load()
     kl = _k_lens_arg(k_lens, B, q.device)
     flags = (_capi.FLAG_PWL_EXP2 if pwl_exp2 else 0) | (_capi.FLAG_SMOOTH_V if smooth_v else 0)
-    if q_lens is not None and (out_dtype is None or out_dtype == q.dtype):
-        out_dtype_eff = q.dtype
-    else:
-        out_dtype_eff = out_dtype
-    if out_dtype_eff is not None and (out_dtype_eff != q.dtype or q_lens is not None):
-        out_dtype = out_dtype_eff
-        if out_dtype not in _DTYPES:
-            raise ValueError(f"out_dtype must be float16 or bfloat16, got {out_dtype}")
-        # the quantized operands carry no dtype: quantize from q's, write the result in the other
+    if prep is not None:
+        _check_qwen_rows(prep, Lq)
+        _check_qwen_rows(prep, k.shape[1])
+    result_dtype = q.dtype if out_dtype is None else out_dtype
+    if result_dtype not in _DTYPES:
+        raise ValueError(f"out_dtype must be float16 or bfloat16, got {out_dtype}")
+    out = torch.empty((B, Lq, Hq, D), dtype=result_dtype, device=q.device)
+    if q_lens is not None or result_dtype != q.dtype:
+        # the one-call entry points take neither q_lens nor a result dtype of their own: quantize (the quantized
+        # operands carry no dtype), then the attention entry point that takes both
         quant_q(q, ws, sm_scale, prep=prep)
         quant_k(k, ws, smooth_k, prep=prep)
         quant_v(v, ws, smooth_v)
-        out = torch.empty((B, Lq, Hq, D), dtype=out_dtype, device=q.device)
         attn_fwd(ws, out, causal=is_causal, pwl_exp2=pwl_exp2, k_lens=kl, block_mask=block_mask, q_lens=q_lens)
         return out.transpose(1, 2) if tensor_layout == "HND" else out
     if block_mask is not None:
@@ -522,9 +525,6 @@ def sageattn(
         )
         _capi.check(rc, "ksana_sage_forward_masked")
         return out.transpose(1, 2) if tensor_layout == "HND" else out
-    if prep is not None:
-        _check_qwen_rows(prep, Lq)
-        _check_qwen_rows(prep, k.shape[1])
     c_prep, _keep = (None, None) if prep is None else prep.to_c(q.device)
     rc = lib.ksana_sage_forward_prep(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), _DTYPES[q.dtype],
