@@ -212,11 +212,15 @@ int ksana_sage_block_means(const void* x, int dtype, const int64_t strides[4], i
                            const float* centre, void* out, void* stream);
 
 /* Did a workgroup of the last ksana_sage_quant_k / ksana_sage_quant_v on this workspace give up waiting for the
- * others of its head?  Both quantizers read their input once: a workgroup keeps its rows in registers while the
+ * others of its head?  Both quantizers can read their input once: a workgroup keeps its rows in registers while the
  * statistic of its head (channel means / column maxima) is gathered from all of them, and that wait is bounded by
- * a two-second limit so that every kernel ends.  On a GPU shared with nothing else the limit is never met; if it is,
- * the status word of the stage is 1 and the quantized operands are not to be used.  SYNCHRONISES `stream`, then
- * copies the two words: a call for tests and diagnostics, not for the hot path.  No counterpart in the reference. */
+ * a two-second limit so that every kernel ends.  On a GPU the call has to itself the limit is never met.  Where it is
+ * (a device shared with other work can hold fewer workgroups at once than the launcher counted on), the workgroup
+ * takes the statistic from the input itself, in the specified order: the quantized operands are the same bits, the
+ * call was slow, and the status word of the stage is 1.  SYNCHRONISES `stream`, then copies the two words: a call
+ * for tests and diagnostics, not for the hot path.  No counterpart in the reference.
+ * (Environment, read at every call: KSANA_SAGE_WAIT_TICKS = the limit in 10 ns ticks, for tests;
+ * KSANA_SAGE_ONE_READ = which of "k", "v" take the one-read kernels when the shape allows, default "v".) */
 int ksana_sage_quant_status(const void* workspace, const ksana_sage_shape* shape, void* stream, int* k_status,
                             int* v_status);
 

@@ -120,13 +120,11 @@ ksana_sage::QuantSync sync_at(int* k_words, int* v_words, int bhk) {
 }
 
 // Which of K and V are quantized by the one-read kernels when the shape allows (otherwise by the two-pass ones):
-// environment variable KSANA_SAGE_ONE_READ = any of the letters "k", "v" ("" = neither); read once.
+// environment variable KSANA_SAGE_ONE_READ = any of the letters "k", "v" ("" = neither; unset = "v"); read at
+// every call.
 bool one_read(char which) {
-  static const char* chosen = [] {
-    const char* e = getenv("KSANA_SAGE_ONE_READ");
-    return e ? e : "v";
-  }();
-  return strchr(chosen, which) != nullptr;
+  const char* e = getenv("KSANA_SAGE_ONE_READ");
+  return strchr(e ? e : "v", which) != nullptr;
 }
 
 int check_ws(const void* ws) {

@@ -362,7 +362,8 @@ def block_means(x: torch.Tensor, rows: int, centre: torch.Tensor | None = None) 
 
 def quant_status(ws: SageWorkspace) -> tuple[int, int]:
     """``(k_status, v_status)`` of the last K / V quantization on ``ws``: 0, or 1 when a workgroup gave up waiting for
-    the others of its head (see ``ksana_sage_quant_status``).  Synchronises the current stream; for tests."""
+    the others of its head and recomputed the head's statistic from the input (same bits, a slow call; see
+    ``ksana_sage_quant_status``).  Synchronises the current stream; for tests."""
     ks, vs = C.c_int(-1), C.c_int(-1)
     rc = _capi.load().ksana_sage_quant_status(ws.ptr, C.byref(ws.shape), _stream_ptr(ws.blob.device), C.byref(ks),
                                               C.byref(vs))

@@ -69,6 +69,37 @@ def test_quantizer_with_prep_is_bit_exact(hip_device, B, L, H, grids, dtype, nor
     _check_k(ws, k_ref, L)
 
 
+@pytest.mark.parametrize("kind", ["wan", "qwen"])
+def test_prep_k_stays_exact_when_a_wait_runs_out(hip_device, kind, monkeypatch):
+    """K with the norm / rotation step folded in always takes the one-read kernel; a workgroup whose bounded wait
+    runs out recomputes the head's mean from the input, norm and rotation included, in the specified order."""
+    monkeypatch.setenv("KSANA_SAGE_WAIT_TICKS", "0")
+    if kind == "wan":
+        B, L, H, grids = 1, 1500, 4, [(5, 10, 30)]
+        kp, wk = _proj(B, L, H, seed=5)
+        table = pr.wan_rope_table(128)
+        prep = WanPrep(q_norm_weight=None, k_norm_weight=wk, eps=1e-6, freqs=table, grid_sizes=grids)
+        k4 = kp.view(B, L, H, 128).to(hip_device)
+        k_ref = pr.wan_prep_ref(kp, wk, 1e-6, grids, table, H)
+    else:
+        B, H, txt, img = 2, 3, 100, 1100
+        L = txt + img
+        g = torch.Generator().manual_seed(17)
+        k = torch.randn((B, L, H, 128), generator=g).bfloat16()
+        w_img = (1.0 + 0.1 * torch.randn(128, generator=g)).float()
+        w_txt = (1.0 + 0.1 * torch.randn(128, generator=g)).float()
+        f_img, f_txt = pr.qwen_rope_table(img, offset=-3), pr.qwen_rope_table(txt, offset=2000)
+        prep = QwenPrep(txt_len=txt, eps=1e-6, k_norm_weight=w_img, k_norm_weight_txt=w_txt, img_freqs=f_img, txt_freqs=f_txt)
+        k4 = k.to(hip_device)
+        k_ref = pr.qwen_prep_ref(k, txt, w_img, w_txt, 1e-6, f_img, f_txt)
+    ws = sage_ops.workspace_for(k4, k4)
+    ws.blob.fill_(0x7F)
+    sage_ops.quant_k(k4, ws, prep=prep)
+    torch.cuda.synchronize()
+    assert sage_ops.quant_status(ws)[0] == 1
+    _check_k(ws, k_ref, L)
+
+
 def test_wan_block_path_equals_attention_on_prepared_tensors(hip_device):
     """norm + RoPE on the fly, then attention == attention fed with the oracle's normed and rotated q, k."""
     B, L, H = 1, 448, 6
