@@ -48,6 +48,15 @@ __device__ __forceinline__ void load_row16(const uint16_t* row_ptr, bool valid, 
   widen8<DT>(b, out + 8);
 }
 
+// 16 bytes of quantizer output.  Non-temporal: the tiles are written once and read next by another kernel, after
+// half a gigabyte of other traffic; stores that do not linger in the caches on their way out measured 6 % off the
+// three quantizers together (405 -> 380 us at B=1 H=40 L=32760), with the attention kernel's time unchanged.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_out16(void* p, uint4 v) {
+  const u32x4 w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(p));
+}
+
 // The same row as it sits in memory (two 16-byte loads), for code that wants the next row in flight while it works
 // on the current one.
 __device__ __forceinline__ void fetch_row16(const uint16_t* row_ptr, bool valid, uint4 (&raw)[2]) {
@@ -576,7 +585,7 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
     const bool nz = amax > 0.0f;
     const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
     if (c16 == 0) q_scale[bh * lq_pad + row] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
-    *reinterpret_cast<uint4*>(q_i8 + (bh * lq_pad + row) * kD + c16 * 16) = pack_int8x16(xr, inv);
+    store_out16(q_i8 + (bh * lq_pad + row) * kD + c16 * 16, pack_int8x16(xr, inv));
   };
   if constexpr (PRE) {
     // The norm and the rotation are arithmetic-heavy (vector fp64): one row at a time with only the next row's two
@@ -657,7 +666,7 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
   for (int i = 0; i < R; ++i) {
     const int frag = i * 4 + (c16 >> 1);
     const int lane = (c16 & 1) * 32 + slot;
-    *reinterpret_cast<uint4*>(tile + (frag * 64 + lane) * 16) = pack_int8x16(x[i], inv);
+    store_out16(tile + (frag * 64 + lane) * 16, pack_int8x16(x[i], inv));
   }
 }
 
@@ -731,7 +740,7 @@ __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __res
       }
       w[g] = acc;
     }
-    *reinterpret_cast<uint4*>(tile + oc * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    store_out16(tile + oc * 16, make_uint4(w[0], w[1], w[2], w[3]));
   }
 }
 
@@ -1044,7 +1053,7 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
     for (int i = 0; i < 2; ++i) {
       const int frag = i * 4 + (c16 >> 1);
       const int ln = (c16 & 1) * 32 + slot;
-      *reinterpret_cast<uint4*>(tile + (frag * 64 + ln) * 16) = pack_int8x16(x[i], inv);
+      store_out16(tile + (frag * 64 + ln) * 16, pack_int8x16(x[i], inv));
     }
   }
 }
@@ -1214,7 +1223,7 @@ __global__ __launch_bounds__(kThreads) void quant_v_fused_kernel(const uint16_t*
         }
         w[g] = a;
       }
-      *reinterpret_cast<uint4*>(tile + oc * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+      store_out16(tile + oc * 16, make_uint4(w[0], w[1], w[2], w[3]));
     }
   }
 }
