@@ -628,7 +628,9 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
                                                            const float* __restrict__ k_mean,
                                                            int8_t* __restrict__ k_tiles, float* __restrict__ k_scale,
                                                            const PrepParams pp) {
-  const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // Heads and batch entries from the last one down: this pass follows the column-sum pass over the same tensor, which
+  // went upwards, so what that pass touched last - and the last-level cache may still hold - is read first.
+  const int blk = blockIdx.x, h = (int)gridDim.y - 1 - (int)blockIdx.y, b = (int)gridDim.z - 1 - (int)blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const int64_t bh = (int64_t)b * H + h;
@@ -682,7 +684,8 @@ __global__ __launch_bounds__(kThreads) void quant_v_kernel(const uint16_t* __res
                                                            const float* __restrict__ v_inv,
                                                            const float* __restrict__ v_mean,
                                                            uint8_t* __restrict__ v_tiles) {
-  const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // (heads and batch entries from the last one down, like quant_k_kernel: the abs-max pass went upwards)
+  const int blk = blockIdx.x, h = (int)gridDim.y - 1 - (int)blockIdx.y, b = (int)gridDim.z - 1 - (int)blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
   const int64_t bh = (int64_t)b * H + h;
