@@ -753,16 +753,35 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // smoothing, and a row that saw no key stays zero
   const float keep_mean = inv_l != 0.0f ? 1.0f : 0.0f;
   constexpr int kPitch = 2 * kD + 16;  // bytes per staged row: 16 bytes of padding spread the rows over the banks
-  __syncthreads();  // waves that ended early (no query rows) do not count
-  uint8_t* stage = smem + wave * (32 * kPitch);
+  // The lane's 16 quadruples of V scales are requested together and ahead of the barrier (the score registers are
+  // free by now); read one quadruple at a time where they are used, every one of the 16 groups below would start
+  // with an LDS round trip of its own.  Without V smoothing the means are all zero - seen here by the wave as a
+  // whole - and their products and sums are left out (a zero output may then keep a minus sign it used to lose).
   const float4* vs4 = reinterpret_cast<const float4*>(s_vs);
   const float4* vm4 = reinterpret_cast<const float4*>(s_vs + kD);
+  float4 s4a[16];
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt) {
+  for (int i = 0; i < 16; ++i) s4a[i] = vs4[(32 * (i >> 2) + 8 * (i & 3) + 4 * hh) >> 2];
+  const float2 mm = reinterpret_cast<const float2*>(s_vs + kD)[lane];
+  const bool has_mean = __any(mm.x != 0.0f || mm.y != 0.0f);  // wave-uniform
+  __syncthreads();  // waves that ended early (no query rows) do not count
+  uint8_t* stage = smem + wave * (32 * kPitch);
+  if (!has_mean) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
+    for (int i = 0; i < 16; ++i) {
+      const int dt = i >> 2, g = i & 3;
       const int d = 32 * dt + 8 * g + 4 * hh;
-      const float4 s4 = vs4[d >> 2];
+      const float4 s4 = s4a[i];
+      *reinterpret_cast<uint2*>(stage + l32 * kPitch + 2 * d) =
+          half4<DT>(oacc[dt][4 * g + 0] * inv_l * s4.x, oacc[dt][4 * g + 1] * inv_l * s4.y,
+                    oacc[dt][4 * g + 2] * inv_l * s4.z, oacc[dt][4 * g + 3] * inv_l * s4.w);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int dt = i >> 2, g = i & 3;
+      const int d = 32 * dt + 8 * g + 4 * hh;
+      const float4 s4 = s4a[i];
       const float4 m4 = vm4[d >> 2];
       *reinterpret_cast<uint2*>(stage + l32 * kPitch + 2 * d) =
           half4<DT>(oacc[dt][4 * g + 0] * inv_l * s4.x + m4.x * keep_mean, oacc[dt][4 * g + 1] * inv_l * s4.y + m4.y * keep_mean,
