@@ -337,10 +337,14 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // the head's K scales (dense: in tile order) and V scales / means go to LDS; without a tile list this waits until
   // the first tile copies are on their way, so that the loads' latencies overlap
   auto fill_scales = [&]() {
+    // the V value is requested first and stored last: written where it is loaded, its load would only go out after
+    // the K scales' loads had been awaited - a second memory latency in every workgroup's set-up
+    float vsm = 0.0f;
+    if (tid < 2 * kD) vsm = tid < kD ? p.v_scale[(int64_t)bhk * kD + tid] : p.v_mean[(int64_t)bhk * kD + tid - kD];
     if constexpr (!kSparse) {
       for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
     }
-    if (tid < 2 * kD) s_vs[tid] = tid < kD ? p.v_scale[(int64_t)bhk * kD + tid] : p.v_mean[(int64_t)bhk * kD + tid - kD];
+    if (tid < 2 * kD) s_vs[tid] = vsm;
   };
   if constexpr (kSparse) fill_scales();
   // Causal calls: the list is in key order, so the entries this wave takes part in (tile <= the one on its diagonal)
