@@ -313,8 +313,7 @@ def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
     def run(e=None):
         if e:
             e[0].record()
-        sage_ops.quant_q(q, ws, sm_scale, prep=prep)
-        sage_ops.quant_k(k, ws, True, prep=prep)
+        sage_ops.quant_qk(q, k, ws, sm_scale, True, prep=prep)
         sage_ops.quant_v(v, ws)
         if e:
             e[1].record()
@@ -353,7 +352,7 @@ def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
     torch.cuda.synchronize()
     eager_ms = e0.elapsed_time(e1)
     return {
-        "what": "row statistic x2 + quantizer with RMSNorm(row of H*D) and 3-axis RoPE on q, k; V as before",
+        "what": "quantizer with RMSNorm(row of H*D) and 3-axis RoPE on q, k (q and k in one call; row statistics taken inside q's kernel); V as before",
         "grid": list(grid),
         "ms": round(ms, 4),
         "bound": "hbm",

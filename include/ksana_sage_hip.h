@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 15
+#define KSANA_SAGE_ABI_VERSION 16
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -186,6 +186,13 @@ int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t q_strides[4]
                             const ksana_sage_prep* prep, float sm_scale, void* workspace, void* stream);
 int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
                             const ksana_sage_prep* prep, int smooth_k, void* workspace, void* stream);
+/* The two calls above as one.  Same results in the same workspace areas; where q's token-row norm makes its kernel
+ * take whole rows anyway, the row statistic of k rides along in that kernel instead of costing a pass over k of its
+ * own.  What a caller that holds q and k together should use (the reference's block does: wan_model.py:163-174,
+ * sage_sla.py:198-204 quantize both in one call). */
+int ksana_sage_quant_qk_prep(const void* q, const void* k, int dtype, const int64_t q_strides[4],
+                             const int64_t k_strides[4], const ksana_sage_shape* shape, const ksana_sage_prep* prep,
+                             float sm_scale, int smooth_k, void* workspace, void* stream);
 
 /* V -> transposed, padded, operand-ordered fp8 e4m3fn with one fp32 scale per (b, h, d).
  * Replaces transpose_pad_permute_cuda + scale_fuse_quant_cuda (sage_sla.py:222-228). */

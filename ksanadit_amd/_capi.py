@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -38,6 +38,7 @@ EXPORTS = (
     "ksana_sage_forward",
     "ksana_sage_quant_q_prep",
     "ksana_sage_quant_k_prep",
+    "ksana_sage_quant_qk_prep",
     "ksana_sage_forward_prep",
     "ksana_sage_attn_fwd_masked",
     "ksana_sage_attn_fwd_varlen",
@@ -113,6 +114,7 @@ def _declare(lib):
     pp = C.POINTER(Prep)
     lib.ksana_sage_quant_q_prep.argtypes, lib.ksana_sage_quant_q_prep.restype = [vp, i, st, sp, pp, f, vp, vp], i
     lib.ksana_sage_quant_k_prep.argtypes, lib.ksana_sage_quant_k_prep.restype = [vp, i, st, sp, pp, i, vp, vp], i
+    lib.ksana_sage_quant_qk_prep.argtypes, lib.ksana_sage_quant_qk_prep.restype = [vp, vp, i, st, st, sp, pp, f, i, vp, vp], i
     lib.ksana_sage_forward_prep.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, pp, vp, f, i, i, i, vp, vp]
     lib.ksana_sage_forward_prep.restype = i
     ms = C.POINTER(C.c_int64)

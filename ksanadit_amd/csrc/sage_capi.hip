@@ -290,8 +290,12 @@ int ksana_sage_quant_q(const void* q, int dtype, const int64_t st[4], const ksan
   return ksana_sage_quant_q_prep(q, dtype, st, s, nullptr, sm_scale, ws, stream);
 }
 
-int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s,
-                            const ksana_sage_prep* prep, float sm_scale, void* ws, void* stream) {
+// `k` != nullptr (the caller has checked k as a tensor): when q's path takes whole token rows anyway (a norm over the
+// row), the row statistic of k is taken along and *k_rms_done says so
+static int quant_q_impl(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s,
+                        const ksana_sage_prep* prep, float sm_scale, void* ws, void* stream, const void* k,
+                        const int64_t k_st[4], bool* k_rms_done) {
+  if (k_rms_done) *k_rms_done = false;
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("q", q, dtype, st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -302,18 +306,30 @@ int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t st[4], const
   if (int rc = make_prep(prep, prep ? prep->q_norm_weight : nullptr, "q", st, s->B, s->Lq, s->D, ws_at<float>(ws, l.q_rms),
                          &pp, &ppp))
     return rc;
-  if (ppp && ppp->inv_rms) {
-    hipError_t e = ksana_sage::launch_row_inv_rms(in_tensor(q, dtype, st), s->B, s->Hq, s->Lq, prep->norm_eps,
-                                                  ws_at<float>(ws, l.q_rms), static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return hip_fail(e, "q row statistic launch");
-  }
   // one fp32 product, then an exact power of two (1/128 undoes the unnormalised Hadamard
   // transforms of Q and K): part of the quantizer specification
   const float premul = (sm_scale * 1.4426950408889634f) * 0.0078125f;
+  if (ppp && ppp->inv_rms) {
+    // a norm over the token row: statistic and quantization in one kernel that takes whole rows
+    const bool take_k = k != nullptr && prep->k_norm_weight != nullptr && k_st[2] == ksana_sage::kD;
+    const ksana_sage::InTensor kt = take_k ? in_tensor(k, dtype, k_st, s->D) : ksana_sage::InTensor{};
+    hipError_t e = ksana_sage::launch_quant_q_rows(in_tensor(q, dtype, st, s->D), s->B, s->Hq, s->Lq, l.lq_pad, premul,
+                                                   prep->norm_eps, ws_at<int8_t>(ws, l.q_i8), ws_at<float>(ws, l.q_scale),
+                                                   static_cast<hipStream_t>(stream), *ppp, take_k ? &kt : nullptr,
+                                                   s->Hkv, s->Lk, ws_at<float>(ws, l.k_rms));
+    if (e != hipSuccess) return hip_fail(e, "quant_q (whole rows) launch");
+    if (k_rms_done) *k_rms_done = take_k;
+    return 0;
+  }
   hipError_t e = ksana_sage::launch_quant_q(in_tensor(q, dtype, st, s->D), s->B, s->Hq, s->Lq, l.lq_pad, premul,
                                             ws_at<int8_t>(ws, l.q_i8), ws_at<float>(ws, l.q_scale),
                                             static_cast<hipStream_t>(stream), ppp);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_q launch");
+}
+
+int ksana_sage_quant_q_prep(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s,
+                            const ksana_sage_prep* prep, float sm_scale, void* ws, void* stream) {
+  return quant_q_impl(q, dtype, st, s, prep, sm_scale, ws, stream, nullptr, nullptr, nullptr);
 }
 
 int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,
@@ -322,9 +338,10 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
 }
 
 // `part` == nullptr: the chunk sums and the counters go to the workspace's own k_part / k_sync areas
+// `rms_done`: the row statistic of k (k_rms area) has been taken by the call before (quant_q_impl)
 static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                         const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, int* sync_words,
-                        void* stream) {
+                        void* stream, bool rms_done = false) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -341,7 +358,7 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
                          &pp, &ppp))
     return rc;
   hipError_t e = hipSuccess;
-  if (ppp && ppp->inv_rms) {
+  if (ppp && ppp->inv_rms && !rms_done) {
     e = ksana_sage::launch_row_inv_rms(kt, s->B, s->Hkv, s->Lk, prep->norm_eps, ws_at<float>(ws, l.k_rms), hs);
     if (e != hipSuccess) return hip_fail(e, "k row statistic launch");
   }
@@ -372,6 +389,24 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
 int ksana_sage_quant_k_prep(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                             const ksana_sage_prep* prep, int smooth_k, void* ws, void* stream) {
   return quant_k_impl(k, dtype, st, s, prep, smooth_k, ws, nullptr, nullptr, stream);
+}
+
+int ksana_sage_quant_qk_prep(const void* q, const void* k, int dtype, const int64_t q_st[4], const int64_t k_st[4],
+                             const ksana_sage_shape* s, const ksana_sage_prep* prep, float sm_scale, int smooth_k,
+                             void* ws, void* stream) {
+  // k is checked before q's kernels go out: nothing is launched for a call that fails
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_tensor("k", k, dtype, k_st, s->B, s->Lk, s->Hkv)) return rc;
+  {
+    ksana_sage::PrepParams pp;
+    const ksana_sage::PrepParams* ppp = nullptr;
+    float dummy = 0.0f;  // only the validation matters here
+    if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", k_st, s->B, s->Lk, s->D, &dummy, &pp, &ppp))
+      return rc;
+  }
+  bool k_rms_done = false;
+  if (int rc = quant_q_impl(q, dtype, q_st, s, prep, sm_scale, ws, stream, k, k_st, &k_rms_done)) return rc;
+  return quant_k_impl(k, dtype, k_st, s, prep, smooth_k, ws, nullptr, nullptr, stream, k_rms_done);
 }
 
 int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,
@@ -590,8 +625,7 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
     if (int rc = make_prep(prep, prep ? prep->k_norm_weight : nullptr, "k", k_st, s->B, s->Lk, s->D, &dummy, &pp, &ppp))
       return rc;
   }
-  if (int rc = ksana_sage_quant_q_prep(q, dtype, q_st, s, prep, sm_scale, ws, stream)) return rc;
-  if (int rc = ksana_sage_quant_k_prep(k, dtype, k_st, s, prep, smooth_k, ws, stream)) return rc;
+  if (int rc = ksana_sage_quant_qk_prep(q, k, dtype, q_st, k_st, s, prep, sm_scale, smooth_k, ws, stream)) return rc;
   if (int rc = ksana_sage_quant_v_smooth(v, dtype, v_st, s, flags & KSANA_SAGE_FLAG_SMOOTH_V, ws, stream)) return rc;
   return ksana_sage_attn_fwd_masked(ws, o, dtype, o_st, s, block_mask, mask_st, k_lens, causal,
                                     flags & ~KSANA_SAGE_FLAG_SMOOTH_V, stream);

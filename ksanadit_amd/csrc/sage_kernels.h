@@ -74,6 +74,12 @@ hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_
                                    hipStream_t s, int* status = nullptr);
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
                           float* q_scale, hipStream_t s, const PrepParams* prep = nullptr);
+// Q with a token-row norm (prep.inv_rms, prep.weight set; kinds 1 and 3): statistic and quantization from one pass over
+// HBM, 32 whole token rows per workgroup; writes prep.inv_rms as launch_row_inv_rms would.  k_rows != nullptr: the
+// statistic of rows [0, k_L) of that tensor (k_H heads of 128 channels, contiguous per row) goes to k_rms on the way.
+hipError_t launch_quant_q_rows(const InTensor& q, int B, int H, int L, int lq_pad, float premul, float eps,
+                               int8_t* q_i8, float* q_scale, hipStream_t s, const PrepParams& prep,
+                               const InTensor* k_rows, int k_H, int k_L, float* k_rms);
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
                           float* k_scale, hipStream_t s, const PrepParams* prep = nullptr);
 // v_mean: nullptr, or the channel means taken off before scaling (V smoothing)

@@ -206,13 +206,14 @@ __device__ __forceinline__ void prep16_qwen(float* x, const PrepParams& pp, int 
 // variant only (with a run-time switch the three variants' table reads add up).
 template <int DT, int KIND>
 __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const RopeLds& rl, int b, int row, int h,
-                                       int c16, bool staged = true) {
+                                       int c16, bool staged = true, const float* row_rms = nullptr) {
   if constexpr (KIND == 2) {
     prep16_qwen<DT>(x, pp, row, c16);
     return;
   }
   if (pp.inv_rms != nullptr) {
-    const float r = pp.inv_rms[(int64_t)b * pp.L + row];
+    // (row_rms: the row's statistic where the caller holds it already, e.g. in LDS)
+    const float r = row_rms != nullptr ? *row_rms : pp.inv_rms[(int64_t)b * pp.L + row];
     const float4* w4 = reinterpret_cast<const float4*>(pp.weight + h * kD + c16 * 16);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -286,14 +287,9 @@ __device__ __forceinline__ RopeLds maybe_stage_rope(const PrepParams& pp, int b,
 // groups of 8 channels i, i+64, i+128, ... in order, adding the 8 squares of each one after the other
 // (fp32, squares of half values are exact); the 64 lane sums meet in an adjacent-pair tree.  The order
 // is part of the result.  grid = (ceil(L / 4), B), 256 threads.
+// the statistic of one row, by one wave (every lane returns it)
 template <int DT>
-__global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
-                                                               int L, int n8, float n_channels, float eps,
-                                                               float* __restrict__ inv_rms) {
-  const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), b = blockIdx.y;
-  if (row >= L) return;
-  const uint16_t* base = x + b * sB + (int64_t)row * sL;
+__device__ __forceinline__ float row_inv_rms_of(const uint16_t* base, int n8, float n_channels, float eps, int lane) {
   float acc = 0.0f;
   for (int g = lane; g < n8; g += 64) {
     float v[8];
@@ -305,7 +301,18 @@ __global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* _
   for (int m = 1; m <= 32; m <<= 1) acc = acc + __shfl_xor(acc, m);
   // sqrtf, not __fsqrt_rn: the latter is the 1-ulp native instruction in this toolchain, the former is
   // correctly rounded (the build passes -fhip-fp32-correctly-rounded-divide-sqrt)
-  if (lane == 0) inv_rms[(int64_t)b * L + row] = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(acc, n_channels) + eps));
+  return __fdiv_rn(1.0f, sqrtf(__fdiv_rn(acc, n_channels) + eps));
+}
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void row_inv_rms_kernel(const uint16_t* __restrict__ x, int64_t sB, int64_t sL,
+                                                               int L, int n8, float n_channels, float eps,
+                                                               float* __restrict__ inv_rms) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), b = blockIdx.y;
+  if (row >= L) return;
+  const float r = row_inv_rms_of<DT>(x + b * sB + (int64_t)row * sL, n8, n_channels, eps, lane);
+  if (lane == 0) inv_rms[(int64_t)b * L + row] = r;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -613,6 +620,111 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) finish_row(x[i], blk * kRowsPerWg + i * kSlots + slot);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Q with a norm over the whole token row folded in (Wan), from ONE pass over HBM.  A workgroup takes 8 whole token
+// rows, all heads.  First their statistics, as row_inv_rms_kernel takes them (one wave per row, two rows per wave,
+// both at a time) - and, where the caller passes k, the statistics of the same rows of k, whose own quantizer then
+// needs no statistic pass of its own.  Then the heads, four at a time: a row slot is (row, one of four heads), 8 lanes
+// x 16 channels each, the next four heads' loads in flight while these are normed, rotated, transformed and packed.
+// The rows are read a second time there, microseconds after the first: from the caches, not from HBM.  Small
+// workgroups on purpose: several generations of them pass through a compute unit, so the memory-bound statistics of
+// some run next to the arithmetic-bound heads of others.
+// grid = (ceil(max(lq_pad, k_L) / 8), B).
+// ---------------------------------------------------------------------------------------
+constexpr int kRowsQ = 8;                   // token rows per workgroup
+constexpr int kHeadsQ = kSlots / kRowsQ;    // heads in work at a time: 4
+struct RowStatOf {  // the rows of another tensor whose statistic the kernel takes along (ptr == nullptr: none)
+  const uint16_t* ptr;
+  int64_t sB, sL;
+  int L, n8;
+  float n_channels;
+  float* inv_rms;  // [B, L]
+};
+
+template <int DT, int KIND>
+__global__ __launch_bounds__(kThreads) void quant_q_rows_kernel(const uint16_t* __restrict__ q, int64_t sB, int64_t sL,
+                                                                int64_t sH, int H, int L, int lq_pad, float premul,
+                                                                float eps, int8_t* __restrict__ q_i8,
+                                                                float* __restrict__ q_scale, const PrepParams pp,
+                                                                float* __restrict__ rms_out, const RowStatOf ks) {
+  const int r0 = blockIdx.x * kRowsQ, b = blockIdx.y;
+  const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
+  const int wave = t >> 6, lane = t & 63;
+  __shared__ float s_rms[kRowsQ];
+  // ---- the rows' statistics: wave w takes rows 2 w and 2 w + 1 together (every row's sum adds its groups of 8
+  // channels in the order of row_inv_rms_of) -------------------------------------------------------------------
+  auto stats = [&](const uint16_t* x, int64_t xsB, int64_t xsL, int xL, int n8, float n_channels, float* out, bool keep) {
+    constexpr int R = kRowsQ / 4;
+    const int first = r0 + wave * R;
+    if (first >= xL) return;  // wave-uniform
+    const uint16_t* rbase = x + b * xsB + (int64_t)first * xsL;
+    float acc[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) acc[i] = 0.0f;
+#pragma unroll 4
+    for (int g = lane; g < n8; g += 64) {
+      uint4 raw[R];
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        raw[i] = first + i < xL ? *reinterpret_cast<const uint4*>(rbase + i * xsL + g * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        float v[8];
+        widen8<DT>(raw[i], v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[i] = acc[i] + v[e] * v[e];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      float a = acc[i];
+#pragma unroll
+      for (int m = 1; m <= 32; m <<= 1) a = a + __shfl_xor(a, m);
+      const float r = __fdiv_rn(1.0f, sqrtf(__fdiv_rn(a, n_channels) + eps));
+      if (lane == 0 && first + i < xL) {
+        out[(int64_t)b * xL + first + i] = r;
+        if (keep) s_rms[wave * R + i] = r;
+      }
+    }
+  };
+  stats(q, sB, sL, L, H * (kD / 8), (float)(H * kD), rms_out, true);
+  if (ks.ptr != nullptr) stats(ks.ptr, ks.sB, ks.sL, ks.L, ks.n8, ks.n_channels, ks.inv_rms, false);
+  if (r0 >= lq_pad) return;  // rows that exist only in k
+  const RopeLds rl = maybe_stage_rope<KIND>(pp, b, r0, kRowsQ);
+  __syncthreads();
+  // ---- the heads, four at a time ------------------------------------------------------------------------------
+  const int rloc = slot & (kRowsQ - 1), h0 = slot / kRowsQ;
+  const int row = r0 + rloc;
+  const bool live = row < L;
+  const uint16_t* base = q + b * sB + (int64_t)row * sL + c16 * 16;
+  uint4 nxt[2];
+  fetch_row16(base + (int64_t)h0 * sH, live && h0 < H, nxt);
+  for (int h = h0; h < H; h += kHeadsQ) {
+    const uint4 cur0 = nxt[0], cur1 = nxt[1];
+    if (h + kHeadsQ < H) fetch_row16(base + (int64_t)(h + kHeadsQ) * sH, live, nxt);
+    float xr[16];
+    widen8<DT>(cur0, xr);
+    widen8<DT>(cur1, xr + 8);
+    if (live) prep16<DT, KIND>(xr, pp, rl, b, row, h, c16, true, &s_rms[rloc]);
+    fwht128(xr, c16);
+    float amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      xr[e] = xr[e] * premul;
+      amax = fmaxf(amax, fabsf(xr[e]));
+    }
+    amax = fmaxf(amax, lane_xor<1>(amax));
+    amax = fmaxf(amax, lane_xor<2>(amax));
+    amax = fmaxf(amax, lane_xor<4>(amax));
+    const bool nz = amax > 0.0f;
+    const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
+    const int64_t bh = (int64_t)b * H + h;
+    if (c16 == 0) q_scale[bh * lq_pad + row] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
+    store_out16(q_i8 + (bh * lq_pad + row) * kD + c16 * 16, pack_int8x16(xr, inv));
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -1397,6 +1509,26 @@ hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, fl
       KSANA_DISPATCH_KIND(pp.kind, (quant_q_kernel<DT, KIND><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, q.D, lq_pad,
                                                                                  premul, q_i8, q_scale, pp)));
     }
+  });
+  return hipGetLastError();
+}
+
+hipError_t launch_quant_q_rows(const InTensor& q, int B, int H, int L, int lq_pad, float premul, float eps,
+                               int8_t* q_i8, float* q_scale, hipStream_t s, const PrepParams& prep,
+                               const InTensor* k_rows, int k_H, int k_L, float* k_rms) {
+  RowStatOf ks{};
+  if (k_rows != nullptr)
+    ks = RowStatOf{k_rows->ptr, k_rows->sB, k_rows->sL, k_L, k_H * (kD / 8), (float)(k_H * kD), k_rms};
+  const int rows = max(lq_pad, k_rows != nullptr ? k_L : 0);
+  const dim3 grid((rows + kRowsQ - 1) / kRowsQ, B), block(kThreads);
+  PrepParams pp = prep;
+  float* rms_out = const_cast<float*>(pp.inv_rms);  // the caller's statistic area: written here, read by nobody else in this launch
+  const size_t lds = plan_rope_lds(&pp, B, kRowsQ);
+  KSANA_DISPATCH_DT(q.dtype, {
+    if (pp.kind == 3)
+      quant_q_rows_kernel<DT, 3><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, eps, q_i8, q_scale, pp, rms_out, ks);
+    else
+      quant_q_rows_kernel<DT, 1><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, eps, q_i8, q_scale, pp, rms_out, ks);
   });
   return hipGetLastError();
 }

@@ -328,6 +328,31 @@ def quant_k(k: torch.Tensor, ws: SageWorkspace, smooth_k: bool = True, prep: "Wa
     _capi.check(rc, "ksana_sage_quant_k")
 
 
+def quant_qk(q: torch.Tensor, k: torch.Tensor, ws: SageWorkspace, sm_scale: float, smooth_k: bool = True,
+             prep: "WanPrep | QwenPrep | None" = None) -> None:
+    """``quant_q`` and ``quant_k`` as one call: the same bits in the same workspace areas.  With a ``prep`` whose norm
+    runs over the whole token row, q's kernel takes whole rows anyway and brings k's row statistic along, which saves
+    k a pass over its input (``ksana_sage_quant_qk_prep``)."""
+    if prep is None:
+        quant_q(q, ws, sm_scale)
+        quant_k(k, ws, smooth_k)
+        return
+    _require_hip(q)
+    _require_hip(k)
+    ws.require(q.device, B=q.shape[0], Lq=q.shape[1], Hq=q.shape[2], D=q.shape[3])
+    ws.require(k.device, B=k.shape[0], Lk=k.shape[1], Hkv=k.shape[2], D=k.shape[3])
+    if k.dtype != q.dtype:
+        raise ValueError("q and k must have the same dtype")
+    q, k = _usable(q), _usable(k)
+    _check_qwen_rows(prep, q.shape[1])
+    _check_qwen_rows(prep, k.shape[1])
+    c_prep, _keep = prep.to_c(q.device)
+    rc = _capi.load().ksana_sage_quant_qk_prep(q.data_ptr(), k.data_ptr(), _DTYPES[q.dtype], _strides(q), _strides(k),
+                                               C.byref(ws.shape), C.byref(c_prep), sm_scale, int(smooth_k), ws.ptr,
+                                               _stream_ptr(q.device))
+    _capi.check(rc, "ksana_sage_quant_qk_prep")
+
+
 def quant_v(v: torch.Tensor, ws: SageWorkspace, smooth_v: bool = False) -> None:
     """``smooth_v``: take the channel means off before scaling; the attention adds them back to its output."""
     _require_hip(v)
@@ -509,8 +534,7 @@ def sageattn(
     if q_lens is not None or result_dtype != q.dtype:
         # the one-call entry points take neither q_lens nor a result dtype of their own: quantize (the quantized
         # operands carry no dtype), then the attention entry point that takes both
-        quant_q(q, ws, sm_scale, prep=prep)
-        quant_k(k, ws, smooth_k, prep=prep)
+        quant_qk(q, k, ws, sm_scale, smooth_k, prep=prep)
         quant_v(v, ws, smooth_v)
         attn_fwd(ws, out, causal=is_causal, pwl_exp2=pwl_exp2, k_lens=kl, block_mask=block_mask, q_lens=q_lens)
         return out.transpose(1, 2) if tensor_layout == "HND" else out

@@ -100,6 +100,30 @@ def test_prep_k_stays_exact_when_a_wait_runs_out(hip_device, kind, monkeypatch):
     _check_k(ws, k_ref, L)
 
 
+@pytest.mark.parametrize("Lq,Lk,Hq,Hkv,grids", [(300, 300, 12, 12, [(3, 9, 11)]), (200, 520, 4, 4, None), (520, 70, 8, 4, None),
+                                                (1000, 1000, 40, 40, [(4, 10, 25)])])
+def test_q_and_k_in_one_call_give_the_bits_of_two(hip_device, Lq, Lk, Hq, Hkv, grids):
+    """``quant_qk``: q's whole-row kernel brings k's row statistic along (k longer than q, shorter, with fewer
+    heads); every workspace area ends up as the two separate calls leave it."""
+    B = 2 if grids is None else 1
+    qp, wq = _proj(B, Lq, Hq, seed=Lq + Hq)
+    kp, wk = _proj(B, Lk, Hkv, seed=Lk + Hkv + 1)
+    table = pr.wan_rope_table(128)
+    prep = WanPrep(q_norm_weight=wq, k_norm_weight=wk, eps=1e-6, freqs=table if grids else None, grid_sizes=grids)
+    q4 = qp.view(B, Lq, Hq, 128).to(hip_device)
+    k4 = kp.view(B, Lk, Hkv, 128).to(hip_device)
+    two, one = sage_ops.workspace_for(q4, k4), sage_ops.workspace_for(q4, k4)
+    two.blob.fill_(0x7F), one.blob.fill_(0x3C)
+    sage_ops.quant_q(q4, two, 128**-0.5, prep=prep)
+    sage_ops.quant_k(k4, two, prep=prep)
+    sage_ops.quant_qk(q4, k4, one, 128**-0.5, prep=prep)
+    torch.cuda.synchronize()
+    assert sage_ops.quant_status(one)[0] == 0
+    for area in ("q_rms", "k_rms", "q_i8", "q_scale", "k_tiles", "k_scale", "k_mean"):
+        assert torch.equal(getattr(one, area).cpu(), getattr(two, area).cpu()), area
+    assert torch.equal(one.k_rms.cpu(), pr.inv_rms_ref(kp, 1e-6))
+
+
 def test_wan_block_path_equals_attention_on_prepared_tensors(hip_device):
     """norm + RoPE on the fly, then attention == attention fed with the oracle's normed and rotated q, k."""
     B, L, H = 1, 448, 6
