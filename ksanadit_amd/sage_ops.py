@@ -16,6 +16,7 @@ import ctypes as C
 from dataclasses import dataclass
 
 import torch
+from torch.utils.weak import WeakTensorKeyDictionary
 
 from . import _capi
 from .layout import TILE_BYTES
@@ -45,6 +46,32 @@ def _usable(t: torch.Tensor) -> torch.Tensor:
                     "strides multiples of 8 and a 16-byte aligned base); further copies are not logged",
                     tuple(t.shape), tuple(s))
     return t.contiguous()
+
+
+_prep_cache = WeakTensorKeyDictionary()  # source tensor -> {(device, dtype): (version, converted)}
+_prep_move_warned = False
+
+
+def _prep_operand(t: torch.Tensor, device, dtype) -> torch.Tensor:
+    """A weight or table of the step before attention as the kernels read it: on ``device``, ``dtype``, contiguous.
+    A conversion is remembered per source tensor (and redone once that tensor has been written to), so a caller that
+    keeps its weights in another dtype - or on the host - pays for it once, not in every attention call; a transfer
+    from another device is logged the first time."""
+    global _prep_move_warned
+    device = torch.device(device)
+    if t.device == device and t.dtype == dtype and t.is_contiguous():
+        return t
+    key = (device, dtype)
+    hit = _prep_cache.get(t, {}).get(key)
+    if hit is not None and hit[0] == t._version:
+        return hit[1]
+    if t.device != device and not _prep_move_warned:
+        _prep_move_warned = True
+        log.warning("Sage HIP path: a norm weight / rotary table lives on %s, the tensors on %s; it is copied over once "
+                    "per tensor (keep them on the device to avoid even that)", t.device, device)
+    conv = t.detach().to(device=device, dtype=dtype).contiguous()
+    _prep_cache.setdefault(t, {})[key] = (t._version, conv)
+    return conv
 
 
 def _stream_ptr(device) -> C.c_void_p:
@@ -184,7 +211,7 @@ class WanPrep:
         def weight(w):
             if w is None:
                 return None
-            w = w.to(device=device, dtype=torch.float32).contiguous()
+            w = _prep_operand(w, device, torch.float32)
             keep.append(w)
             return w.data_ptr()
 
@@ -199,7 +226,7 @@ class WanPrep:
                 m = m[0, :, 0]
             if m.dim() != 4 or tuple(m.shape[1:]) != (64, 2, 2) or m.is_complex():
                 raise ValueError(f"comfy_freqs must be [1, rows, 1, 64, 2, 2] or [rows, 64, 2, 2], got {tuple(self.comfy_freqs.shape)}")
-            m = m.to(device=device, dtype=torch.float32).contiguous()
+            m = _prep_operand(m, device, torch.float32)
             keep.append(m)
             c.kind = _capi.PREP_WAN_COMFY
             c.rope_matrices, c.rope_rows = m.data_ptr(), m.shape[0]
@@ -208,7 +235,7 @@ class WanPrep:
                 raise ValueError("freqs must be a complex [rows, D/2] tensor")
             if self.grid_sizes is None:
                 raise ValueError("freqs given without grid_sizes")
-            fr = self.freqs.to(device=device, dtype=torch.complex128).contiguous()
+            fr = _prep_operand(self.freqs, device, torch.complex128)
             grid = torch.as_tensor(self.grid_sizes).to(device="cpu", dtype=torch.int32).contiguous()
             if grid.dim() != 2 or grid.shape[1] != 3:
                 raise ValueError(f"grid_sizes must be [B, 3], got {tuple(grid.shape)}")
@@ -243,7 +270,7 @@ class QwenPrep:
         def weight(w):
             if w is None:
                 return None
-            w = w.to(device=device, dtype=torch.float32).contiguous()
+            w = _prep_operand(w, device, torch.float32)
             if w.numel() != 128:
                 raise ValueError("Qwen norm weights are per head channel: 128 values")
             keep.append(w)
@@ -256,7 +283,7 @@ class QwenPrep:
                 raise ValueError("rotary tables must be complex [rows, 64]")
             if t.shape[0] < rows:
                 raise ValueError(f"rotary table has {t.shape[0]} rows, the segment {rows}")
-            t = torch.view_as_real(t.to(device=device, dtype=torch.complex64).contiguous())
+            t = torch.view_as_real(_prep_operand(t, device, torch.complex64))
             keep.append(t)
             return t.data_ptr()
 

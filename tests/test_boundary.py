@@ -316,3 +316,22 @@ def test_workload_table():
     qo, ko, _ = make_inputs("wan14b_480p", heads=1, seq=4096)
     assert qo.float().abs().max() > 20 and ko.float().abs().max() > 20  # x20 outliers present
     assert ksanadit_amd.DEFAULT_ATTENTION_BACKEND == KsanaAttentionBackend.SAGE_ATTN
+
+
+def test_prep_operands_are_converted_once_per_source_tensor():
+    """Norm weights and rotary tables that are not in the kernels' dtype (or not on the device) are converted on first
+    use and the result is reused until the source tensor is written to."""
+    from ksanadit_amd import sage_ops
+
+    w = torch.randn(128, dtype=torch.bfloat16)
+    a = sage_ops._prep_operand(w, "cpu", torch.float32)
+    assert a.dtype == torch.float32 and torch.equal(a, w.float())
+    assert sage_ops._prep_operand(w, "cpu", torch.float32) is a
+    w.mul_(2.0)
+    b = sage_ops._prep_operand(w, "cpu", torch.float32)
+    assert b is not a and torch.equal(b, w.float())
+    ready = torch.randn(128)
+    assert sage_ops._prep_operand(ready, "cpu", torch.float32) is ready  # nothing to convert: passed through
+    table = torch.polar(torch.ones(8, 64), torch.randn(8, 64))  # complex64
+    t128 = sage_ops._prep_operand(table, "cpu", torch.complex128)
+    assert t128.dtype == torch.complex128 and sage_ops._prep_operand(table, "cpu", torch.complex128) is t128
