@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 16
+#define KSANA_SAGE_ABI_VERSION 17
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -152,6 +152,29 @@ typedef struct ksana_sage_prep {
 int ksana_sage_abi_version(void);
 const char* ksana_sage_last_error(void);
 
+/* Process-wide settings of the one-read K / V quantizers (see ksana_sage_quant_status for what they are).  No
+ * counterpart in the reference.
+ *   one_read_stages: NULL = leave as it is; otherwise a string of the letters "k" and "v": the stages that take the
+ *     one-read kernel when the shape allows ("" = neither).  First value: the environment variable
+ *     KSANA_SAGE_ONE_READ, default "v"; the environment is read once, when the first call needs it.  K with a folded
+ *     norm / rotation step always tries the one-read kernel.
+ *   wait_ticks: KSANA_SAGE_KEEP = leave as it is; otherwise the bound, in 10 ns ticks, on a workgroup's wait for its
+ *     head's statistic.  First value: KSANA_SAGE_WAIT_TICKS, default 200000 (2 ms; the kernels run 0.1 - 0.5 ms).
+ *     A positive bound that expires makes the library take the two-pass kernels on that GPU from the next call on (the
+ *     GPU evidently holds fewer workgroups at once than the launcher counted on, e.g. because it is shared; results
+ *     are the same bits either way).  0 (give up at the first poll that finds the flag down) and negative values (do
+ *     not poll: every workgroup but a head's last arriver recomputes the statistic from the input) exercise that path
+ *     in tests and switch nothing off.
+ * Every call also re-arms the one-read kernels on all GPUs. */
+#define KSANA_SAGE_KEEP INT64_MIN
+int ksana_sage_configure(const char* one_read_stages, int64_t wait_ticks);
+/* The current settings, and whether the one-read kernels are switched off on the current GPU because a wait expired
+ * there (any out-pointer may be NULL).  Reads host memory only; for logs and tests. */
+int ksana_sage_one_read_state(int* one_read_k, int* one_read_v, int64_t* wait_ticks, int* demoted);
+/* Host-side self-checks of the library's bookkeeping (today: that two instantiations of one kernel template keep
+ * separate entries in the cache of resident-workgroup counts).  Touches no device; 0 = all passed. */
+int ksana_sage_selftest(void);
+
 /* Size/offsets of the scratch the stages below share.  Replaces the torch.empty calls the
  * reference makes for its quantized operands (sage_sla.py:222-227). */
 int ksana_sage_workspace_layout(const ksana_sage_shape* shape, ksana_sage_ws_layout* out);
@@ -173,7 +196,11 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t k_strides[4], con
  * per-256-row chunk sums behind the channel means) lives: not in the workspace's k_part area, which this call
  * leaves untouched, but in a 9 MiB array inside the library's own device image.  Limits: B * Hkv * ceil(Lk / 256)
  * <= 16384 and B * Hkv <= 4096 (KSANA_SAGE_ENOTSUP beyond).  The call allocates and frees nothing.  All calls on one GPU share that
- * array: calls that overlap on one GPU (different streams or threads) race and must be ordered by the caller. */
+ * array: calls that overlap on one GPU (different streams or threads) race and must be ordered by the caller.
+ * Under graph capture: make one ordinary call on the device first (the first call looks the array's address up and
+ * may load the code object, which a capturing stream can refuse).  The counters through which the workgroups of the
+ * one-read kernel meet (KSANA_SAGE_ONE_READ=k) live in that array too: ksana_sage_quant_status, which reads the
+ * workspace's words, says nothing about this call. */
 int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t k_strides[4], const ksana_sage_shape* shape,
                               int smooth_k, void* workspace, void* stream);
 
@@ -221,13 +248,11 @@ int ksana_sage_block_means(const void* x, int dtype, const int64_t strides[4], i
 /* Did a workgroup of the last ksana_sage_quant_k / ksana_sage_quant_v on this workspace give up waiting for the
  * others of its head?  Both quantizers can read their input once: a workgroup keeps its rows in registers while the
  * statistic of its head (channel means / column maxima) is gathered from all of them, and that wait is bounded by
- * a two-second limit so that every kernel ends.  On a GPU the call has to itself the limit is never met.  Where it is
+ * a limit (2 ms by default, ksana_sage_configure) so that every kernel ends.  On a GPU the call has to itself the limit is never met.  Where it is
  * (a device shared with other work can hold fewer workgroups at once than the launcher counted on), the workgroup
  * takes the statistic from the input itself, in the specified order: the quantized operands are the same bits, the
  * call was slow, and the status word of the stage is 1.  SYNCHRONISES `stream`, then copies the two words: a call
- * for tests and diagnostics, not for the hot path.  No counterpart in the reference.
- * (Environment, read at every call: KSANA_SAGE_WAIT_TICKS = the limit in 10 ns ticks, for tests;
- * KSANA_SAGE_ONE_READ = which of "k", "v" take the one-read kernels when the shape allows, default "v".) */
+ * for tests and diagnostics, not for the hot path.  No counterpart in the reference. */
 int ksana_sage_quant_status(const void* workspace, const ksana_sage_shape* shape, void* stream, int* k_status,
                             int* v_status);
 

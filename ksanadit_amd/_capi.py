@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -20,10 +20,14 @@ FLAG_SMOOTH_V = 2
 FLAG_WG_4_WAVES = 4
 FLAG_WG_8_WAVES = 8
 PREP_WAN, PREP_WAN_COMFY, PREP_QWEN = 0, 1, 2
+KEEP = -(2**63)  # KSANA_SAGE_KEEP
 
 EXPORTS = (
     "ksana_sage_abi_version",
     "ksana_sage_last_error",
+    "ksana_sage_configure",
+    "ksana_sage_one_read_state",
+    "ksana_sage_selftest",
     "ksana_sage_workspace_layout",
     "ksana_sage_quant_q",
     "ksana_sage_quant_k",
@@ -96,6 +100,10 @@ def _declare(lib):
     lib.ksana_sage_abi_version.argtypes, lib.ksana_sage_abi_version.restype = [], i
     lib.ksana_sage_last_error.argtypes, lib.ksana_sage_last_error.restype = [], C.c_char_p
     lib.ksana_sage_workspace_layout.argtypes, lib.ksana_sage_workspace_layout.restype = [sp, lp], i
+    lib.ksana_sage_configure.argtypes, lib.ksana_sage_configure.restype = [C.c_char_p, C.c_int64], i
+    lib.ksana_sage_one_read_state.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int64), C.POINTER(C.c_int)]
+    lib.ksana_sage_one_read_state.restype = i
+    lib.ksana_sage_selftest.argtypes, lib.ksana_sage_selftest.restype = [], i
     lib.ksana_sage_quant_q.argtypes, lib.ksana_sage_quant_q.restype = [vp, i, st, sp, f, vp, vp], i
     lib.ksana_sage_quant_k.argtypes, lib.ksana_sage_quant_k.restype = [vp, i, st, sp, i, vp, vp], i
     lib.ksana_sage_quant_k_static.argtypes, lib.ksana_sage_quant_k_static.restype = [vp, i, st, sp, i, vp, vp], i

@@ -119,12 +119,11 @@ ksana_sage::QuantSync sync_at(int* k_words, int* v_words, int bhk) {
   return q;
 }
 
-// Which of K and V are quantized by the one-read kernels when the shape allows (otherwise by the two-pass ones):
-// environment variable KSANA_SAGE_ONE_READ = any of the letters "k", "v" ("" = neither; unset = "v"); read at
-// every call.
+// Which of K and V are quantized by the one-read kernels when the shape allows (otherwise by the two-pass ones): a
+// process-wide setting (ksana_sage_configure; first value from the environment, read once)
 bool one_read(char which) {
-  const char* e = getenv("KSANA_SAGE_ONE_READ");
-  return strchr(e ? e : "v", which) != nullptr;
+  const ksana_sage::QuantOptions o = ksana_sage::quant_options();
+  return which == 'k' ? o.one_read_k : o.one_read_v;
 }
 
 int check_ws(const void* ws) {
@@ -246,6 +245,28 @@ int ksana_sage_abi_version(void) { return KSANA_SAGE_ABI_VERSION; }
 
 const char* ksana_sage_last_error(void) { return g_err; }
 
+int ksana_sage_configure(const char* one_read_stages, int64_t wait_ticks) {
+  if (one_read_stages != nullptr)
+    for (const char* c = one_read_stages; *c; ++c)
+      if (*c != 'k' && *c != 'v') return fail(KSANA_SAGE_EINVAL, "one_read_stages \"%s\": letters k and v only", one_read_stages);
+  ksana_sage::configure_quant(one_read_stages, wait_ticks, wait_ticks == KSANA_SAGE_KEEP);
+  return 0;
+}
+
+int ksana_sage_one_read_state(int* one_read_k, int* one_read_v, int64_t* wait_ticks, int* demoted) {
+  const ksana_sage::QuantOptions o = ksana_sage::quant_options();
+  if (one_read_k) *one_read_k = o.one_read_k;
+  if (one_read_v) *one_read_v = o.one_read_v;
+  if (wait_ticks) *wait_ticks = o.wait_ticks;
+  if (demoted) *demoted = ksana_sage::one_read_demoted(/*may_allocate=*/false) ? 1 : 0;
+  return 0;
+}
+
+int ksana_sage_selftest(void) {
+  const int rc = ksana_sage::selftest_occupancy_cache();
+  return rc == 0 ? 0 : fail(KSANA_SAGE_EINVAL, "occupancy cache self-check failed at step %d", rc);
+}
+
 int ksana_sage_workspace_layout(const ksana_sage_shape* s, ksana_sage_ws_layout* out) {
   if (int rc = check_shape(s)) return rc;
   if (!out) return fail(KSANA_SAGE_EINVAL, "layout out-pointer is null");
@@ -341,7 +362,7 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
 // `rms_done`: the row statistic of k (k_rms area) has been taken by the call before (quant_q_impl)
 static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                         const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, int* sync_words,
-                        void* stream, bool rms_done = false) {
+                        void* stream, bool rms_done = false, bool may_allocate = true) {
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -370,7 +391,8 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
     bool used = false;
     e = ksana_sage::launch_quant_k_fused(kt, s->B, s->Hkv, s->Lk, l.nkb, l.nch, smooth_k ? 1 : 0, part,
                                          ws_at<float>(ws, l.k_mean), ws_at<int8_t>(ws, l.k_i8),
-                                         ws_at<float>(ws, l.k_scale), sync_at(sync_words, nullptr, bhk), hs, ppp, &used);
+                                         ws_at<float>(ws, l.k_scale), sync_at(sync_words, nullptr, bhk), hs, ppp, &used,
+                                         may_allocate);
     if (e != hipSuccess) return hip_fail(e, "fused quant_k launch");
     if (used) return 0;
   }
@@ -426,7 +448,7 @@ int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t st[4], con
   // every chunk sum that is read is written earlier in the same call; the counters and flags behind the partial
   // sums are cleared by the call's first kernel
   return quant_k_impl(k, dtype, st, s, nullptr, smooth_k, ws, part, reinterpret_cast<int*>(part + kStaticPartFloats),
-                      stream);
+                      stream, false, /*may_allocate=*/false);
 }
 
 int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, void* ws,

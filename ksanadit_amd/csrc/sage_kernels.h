@@ -99,10 +99,37 @@ struct QuantSync {
   int* v_status;   // a wait that ran into its limit
 };
 hipError_t launch_clear_ints(int* p, int n, hipStream_t s);
+
+// Process-wide settings of the one-read quantizers.  Their first values come from the environment, read once when
+// the first call needs them (KSANA_SAGE_ONE_READ: which of "k", "v" take the one-read kernels when the shape allows,
+// default "v"; KSANA_SAGE_WAIT_TICKS: the bound below); configure_quant replaces them.
+constexpr long long kDefaultWaitTicks = 200000;  // 2 ms at 100 MHz: ten to twenty times a healthy kernel's whole run
+struct QuantOptions {
+  bool one_read_k, one_read_v;
+  // Wall-clock ticks (10 ns) a workgroup waits for its head's statistic before it takes it from the input itself.
+  // > 0: a bound for production; an expiry also switches the one-read kernels off on that device (see
+  // one_read_demoted).  0: give up at the first poll that finds the flag down; < 0: do not look at the flag at all,
+  // every workgroup but the head's last arriver recomputes - both are for tests and switch nothing off.
+  long long wait_ticks;
+};
+QuantOptions quant_options();
+// stages == nullptr / keep_ticks: leave that setting as it is.  Also forgets every device's demotion.
+void configure_quant(const char* stages, long long wait_ticks, bool keep_ticks);
+// Has a workgroup's wait run into a bound > 0 on the current device since the last configure_quant?  The launchers
+// then take the two-pass kernels there: a device that holds fewer workgroups than its occupancy figure promises
+// (shared with other work) would pay the bound in every call.  `may_allocate` == false never creates the
+// host-visible word the kernels report through (for callers that must not allocate): without it nothing is
+// reported and the answer is false.
+bool one_read_demoted(bool may_allocate = true);
+// 0 when two kernel instantiations of one function-pointer type keep separate entries in the launchers' cache of
+// resident-workgroup counts (a host-side self-check; touches no device)
+int selftest_occupancy_cache();
+
 // One-read quantizers: *used == false means the shape does not suit them and nothing was launched.
+// `may_allocate`: see one_read_demoted.
 hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb, int nch, int smooth, float* part,
                                 float* k_mean, int8_t* k_tiles, float* k_scale, const QuantSync& sync, hipStream_t s,
-                                const PrepParams* prep, bool* used);
+                                const PrepParams* prep, bool* used, bool may_allocate = true);
 hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb, int nch, float* part, float* v_scale,
                                 float* v_inv, float* v_mean, uint8_t* v_tiles, const QuantSync& sync, hipStream_t s,
                                 bool* used);

@@ -8,8 +8,9 @@
 // specification): plain IEEE fp32 add / sub / mul / div, round-half-even, no contraction.
 #include "sage_kernels.h"
 
-#include <atomic>
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
 
 #include "../../include/ksana_sage_hip.h"
 
@@ -927,22 +928,37 @@ __device__ __forceinline__ void publish_f32(float* p, float v) {
 // has reached the point of coherence - and the compiler moves no access across
 __device__ __forceinline__ void complete_accesses() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
 
-// Thread 0 waits until *flag reaches `want` (or the time limit passes), then the workgroup meets.  Returns true
-// (to every thread) when the limit passed first.
-__device__ __forceinline__ bool wait_for_head(const int* flag, int want, long long limit_ticks, int* status) {
+struct HeadSync {
+  int* counter;      // [B*H][kSyncStride] chunks counted in (one word per head, each in a cache line of its own)
+  int* ready;        // [B*H][kSyncStride] set once the head's statistic is published
+  int* status;       // [1]   set to 1 when a wait ran into its time limit
+  long long limit;   // wall-clock ticks (100 MHz) a workgroup waits at most; 0 and negative: see QuantOptions
+  int* host_word;    // nullptr, or a word in host memory the device can write: set to 1 when a bound > 0 expires
+};
+
+// Thread 0 waits until the head's ready flag is up (or the time limit passes), then the workgroup meets.  Returns
+// true (to every thread) when the workgroup has to take the statistic from the input itself: the limit passed first,
+// or the limit is negative, which means "do not even look".
+__device__ __forceinline__ bool wait_for_head(const int* flag, const HeadSync& sy) {
   __shared__ int s_gave_up;
   if (threadIdx.x == 0) {
     int gave_up = 0;
-    if (load_shared_i32(flag) < want) {
+    if (sy.limit < 0) {
+      gave_up = 1;
+    } else if (load_shared_i32(flag) < 1) {
       const long long t0 = wall_clock64();
-      while (load_shared_i32(flag) < want) {
+      while (load_shared_i32(flag) < 1) {
         __builtin_amdgcn_s_sleep(16);  // ~0.5 us between polls
-        if (wall_clock64() - t0 > limit_ticks) {
-          __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (wall_clock64() - t0 > sy.limit) {
           gave_up = 1;
           break;
         }
       }
+    }
+    if (gave_up) {
+      __hip_atomic_store(sy.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (sy.limit > 0 && sy.host_word != nullptr)
+        __hip_atomic_store(sy.host_word, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     s_gave_up = gave_up;
     complete_accesses();
@@ -950,13 +966,6 @@ __device__ __forceinline__ bool wait_for_head(const int* flag, int want, long lo
   __syncthreads();
   return s_gave_up != 0;
 }
-
-struct HeadSync {
-  int* counter;      // [B*H][kSyncStride] chunks counted in (one word per head, each in a cache line of its own)
-  int* ready;        // [B*H][kSyncStride] set once the head's statistic is published
-  int* status;       // [1]   set to 1 when a wait ran into its time limit
-  long long limit;   // wall-clock ticks (100 MHz) a workgroup waits at most
-};
 
 // Staging of one head's chunk partials for the workgroup that combines them: kFinStage chunks per
 // pass (16 KiB of LDS), fetched with loads that are all in flight together; the next pass is fetched while this one
@@ -1092,7 +1101,7 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
     if (t == 0) __hip_atomic_store(sy.ready + bh * kSyncStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   } else {
     // ---- 3. everybody else waits for it -----------------------------------------------------------
-    if (!wait_for_head(sy.ready + bh * kSyncStride, 1, sy.limit, sy.status)) {
+    if (!wait_for_head(sy.ready + bh * kSyncStride, sy)) {
       if (t < kD) s_mean[t] = load_shared_f32(k_mean + bh * kD + t);
       __syncthreads();
     } else {
@@ -1259,7 +1268,7 @@ __global__ __launch_bounds__(kThreads) void quant_v_fused_kernel(const uint16_t*
     __syncthreads();
     if (t == 0) __hip_atomic_store(sy.ready + bh * kSyncStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   } else {
-    if (!wait_for_head(sy.ready + bh * kSyncStride, 1, sy.limit, sy.status)) {
+    if (!wait_for_head(sy.ready + bh * kSyncStride, sy)) {
       if (t < kD) s_inv[t] = load_shared_f32(v_inv + bh * kD + t);
       __syncthreads();
     } else {
@@ -1552,38 +1561,155 @@ hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const
 }
 
 namespace {
+constexpr int kMaxDevices = 64;
+
+// Resident-workgroup counts the launchers have asked the runtime for, kept per (device, kernel address): every
+// instantiation of a kernel template has its own register and LDS footprint, and all instantiations of one
+// template share one function-pointer TYPE, so the address is the key.
+class OccupancyCache {
+ public:
+  int find(int dev, const void* kernel) {
+    std::lock_guard<std::mutex> lock(m_);
+    for (int i = 0; i < n_; ++i)
+      if (e_[i].dev == dev && e_[i].kernel == kernel) return e_[i].workgroups;
+    return -1;
+  }
+  void put(int dev, const void* kernel, int workgroups) {
+    std::lock_guard<std::mutex> lock(m_);
+    for (int i = 0; i < n_; ++i)
+      if (e_[i].dev == dev && e_[i].kernel == kernel) {
+        e_[i].workgroups = workgroups;
+        return;
+      }
+    if (n_ < kEntries) e_[n_++] = Entry{dev, kernel, workgroups};  // full: the answer is simply asked for again
+  }
+
+ private:
+  struct Entry {
+    int dev;
+    const void* kernel;
+    int workgroups;
+  };
+  static constexpr int kEntries = 256;
+  std::mutex m_;
+  Entry e_[kEntries];
+  int n_ = 0;
+};
+OccupancyCache g_occupancy;
+
 // Workgroups of `kernel` (256 threads, `lds` bytes of dynamic LDS) the current device holds at once.
 // (0 when the runtime cannot tell: the caller then takes the two-pass kernels.)  The answer for a launch
 // without dynamic LDS is kept per device and kernel.
 template <typename K>
 int resident_workgroups(K kernel, size_t lds) {
-  constexpr int kMaxDevices = 64;
-  static std::atomic<int> cached[kMaxDevices];
   int per_cu = 0, dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  const void* key = reinterpret_cast<const void*>(kernel);
   if (lds == 0) {
-    const int c = cached[dev].load(std::memory_order_acquire);
+    const int c = g_occupancy.find(dev, key);
     if (c > 0) return c;
   }
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds) != hipSuccess) return 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (lds == 0) cached[dev].store(per_cu * cus, std::memory_order_release);
+  if (lds == 0 && per_cu * cus > 0) g_occupancy.put(dev, key, per_cu * cus);
   return per_cu * cus;
 }
-// Wall-clock ticks (100 MHz) a workgroup waits for its head: 2 s, or what the environment variable
-// KSANA_SAGE_WAIT_TICKS says (read at every call; 0 makes every waiting workgroup take the statistic from the input
-// itself, which is how the tests reach that path).
-long long wait_limit_ticks() {
-  const char* e = getenv("KSANA_SAGE_WAIT_TICKS");
-  if (e != nullptr && *e != 0) {
+
+// ---- process-wide settings (see QuantOptions) ----------------------------------------------------------------
+std::mutex g_opt_mutex;
+bool g_opt_ready = false;
+QuantOptions g_opt{false, true, kDefaultWaitTicks};
+
+void parse_stages(const char* stages, QuantOptions* o) {
+  o->one_read_k = strchr(stages, 'k') != nullptr;
+  o->one_read_v = strchr(stages, 'v') != nullptr;
+}
+void options_from_environment_locked() {
+  if (g_opt_ready) return;
+  g_opt_ready = true;
+  const char* e = getenv("KSANA_SAGE_ONE_READ");
+  parse_stages(e ? e : "v", &g_opt);
+  const char* w = getenv("KSANA_SAGE_WAIT_TICKS");
+  if (w != nullptr && *w != 0) {
     char* end = nullptr;
-    const long long v = strtoll(e, &end, 10);
-    if (end != e && v >= 0) return v;
+    const long long v = strtoll(w, &end, 10);
+    if (end != w) g_opt.wait_ticks = v;
   }
-  return 200000000;
+}
+
+// One word of host memory per device that the device can write (pinned, mapped): a kernel whose wait expires sets it,
+// the launchers read it as plain host memory - no copy, no synchronisation.  Allocated when a one-read kernel is first
+// launched on the device by a caller that may allocate, and kept until the process ends.
+struct HostWord {
+  int* host = nullptr;
+  int* dev = nullptr;
+};
+HostWord g_host_word[kMaxDevices];
+std::mutex g_host_word_mutex;
+
+HostWord host_word(bool may_allocate) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return HostWord{};
+  std::lock_guard<std::mutex> lock(g_host_word_mutex);
+  HostWord& w = g_host_word[dev];
+  if (w.host == nullptr && may_allocate) {
+    void* h = nullptr;
+    void* d = nullptr;
+    if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess) {
+      *static_cast<volatile int*>(h) = 0;
+      if (hipHostGetDevicePointer(&d, h, 0) == hipSuccess) {
+        w.host = static_cast<int*>(h);
+        w.dev = static_cast<int*>(d);
+      } else {
+        (void)hipGetLastError();
+        (void)hipHostFree(h);
+      }
+    } else {
+      (void)hipGetLastError();  // no word, no reports: the kernels still end and still give the same bits
+    }
+  }
+  return w;
 }
 
 }  // namespace
+
+QuantOptions quant_options() {
+  std::lock_guard<std::mutex> lock(g_opt_mutex);
+  options_from_environment_locked();
+  return g_opt;
+}
+
+void configure_quant(const char* stages, long long wait_ticks, bool keep_ticks) {
+  {
+    std::lock_guard<std::mutex> lock(g_opt_mutex);
+    options_from_environment_locked();
+    if (stages != nullptr) parse_stages(stages, &g_opt);
+    if (!keep_ticks) g_opt.wait_ticks = wait_ticks;
+  }
+  std::lock_guard<std::mutex> lock(g_host_word_mutex);
+  for (HostWord& w : g_host_word)
+    if (w.host != nullptr) *static_cast<volatile int*>(w.host) = 0;
+}
+
+bool one_read_demoted(bool may_allocate) {
+  const HostWord w = host_word(may_allocate);
+  return w.host != nullptr && *static_cast<volatile int*>(w.host) != 0;
+}
+
+int selftest_occupancy_cache() {
+  OccupancyCache c;
+  const void* a = reinterpret_cast<const void*>(&quant_k_fused_kernel<KSANA_SAGE_BF16, 1>);
+  const void* b = reinterpret_cast<const void*>(&quant_k_fused_kernel<KSANA_SAGE_BF16, 2>);
+  if (a == b) return 1;
+  if (c.find(0, a) != -1) return 2;
+  c.put(0, a, 768);
+  if (c.find(0, a) != 768 || c.find(0, b) != -1 || c.find(1, a) != -1) return 3;
+  c.put(0, b, 1024);
+  c.put(1, a, 512);
+  if (c.find(0, a) != 768 || c.find(0, b) != 1024 || c.find(1, a) != 512) return 4;
+  c.put(0, a, 256);
+  return c.find(0, a) == 256 && c.find(0, b) == 1024 ? 0 : 5;
+}
 
 hipError_t launch_block_means(const InTensor& x, int B, int H, int L, int rows, const float* centre, uint16_t* out,
                               hipStream_t s) {
@@ -1602,11 +1728,12 @@ hipError_t launch_clear_ints(int* p, int n, hipStream_t s) {
 // comment above the kernels); *used tells the caller whether anything was launched.
 hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb, int nch, int smooth, float* part,
                                 float* k_mean, int8_t* k_tiles, float* k_scale, const QuantSync& sync, hipStream_t s,
-                                const PrepParams* prep, bool* used) {
+                                const PrepParams* prep, bool* used, bool may_allocate) {
   *used = false;
   if ((int64_t)B * H * nch > INT32_MAX) return hipSuccess;
+  if (one_read_demoted(may_allocate)) return hipSuccess;
   const dim3 grid(B * H * nch), block(kThreads);
-  const HeadSync sy{sync.k_counter, sync.k_ready, sync.k_status, wait_limit_ticks()};
+  const HeadSync sy{sync.k_counter, sync.k_ready, sync.k_status, quant_options().wait_ticks, host_word(false).dev};
   const PrepParams none{};
   hipError_t e = hipSuccess;
   KSANA_DISPATCH_DT(k.dtype, {
@@ -1621,7 +1748,7 @@ hipError_t launch_quant_k_fused(const InTensor& k, int B, int H, int L, int nkb,
       PrepParams pp = *prep;
       const size_t lds = plan_rope_lds(&pp, B, kMeanChunk);
       KSANA_DISPATCH_KIND(pp.kind, {
-        // lds != 0 only for kind 1; the cached answer (lds == 0) is kept per instantiation
+        // lds != 0 only for kind 1; the cached answer (lds == 0) is kept per kernel address
         if (2 * nch <= resident_workgroups(quant_k_fused_kernel<DT, KIND>, lds)) {
           quant_k_fused_kernel<DT, KIND><<<grid, block, lds, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb, nch, part, k_mean,
                                                                    k.dtype, smooth, k_tiles, k_scale, pp, sy);
@@ -1639,8 +1766,9 @@ hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb,
                                 bool* used) {
   *used = false;
   if ((int64_t)B * H * nch > INT32_MAX) return hipSuccess;
+  if (one_read_demoted()) return hipSuccess;
   const dim3 grid(B * H * nch), block(kThreads);
-  const HeadSync sy{sync.v_counter, sync.v_ready, sync.v_status, wait_limit_ticks()};
+  const HeadSync sy{sync.v_counter, sync.v_ready, sync.v_status, quant_options().wait_ticks, host_word(false).dev};
   hipError_t e = hipSuccess;
   KSANA_DISPATCH_DT(v.dtype, {
     const int resident = resident_workgroups(quant_v_fused_kernel<DT>, 0);

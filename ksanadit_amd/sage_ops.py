@@ -423,6 +423,40 @@ def quant_status(ws: SageWorkspace) -> tuple[int, int]:
     return ks.value, vs.value
 
 
+def configure(one_read: str | None = None, wait_ticks: int | None = None) -> None:
+    """Process-wide settings of the one-read K / V quantizers (``ksana_sage_configure``): ``one_read`` is a string of
+    the letters ``k`` and ``v`` (the stages that read their input once when the shape allows), ``wait_ticks`` the bound
+    on a workgroup's wait for its head's statistic in 10 ns ticks (0 / negative: test modes, see the header).
+    ``None`` leaves a setting as it is.  Every call re-arms the one-read kernels on all GPUs."""
+    rc = _capi.load().ksana_sage_configure(None if one_read is None else one_read.encode(),
+                                           _capi.KEEP if wait_ticks is None else int(wait_ticks))
+    _capi.check(rc, "ksana_sage_configure")
+
+
+def one_read_state() -> dict:
+    """``{"k": bool, "v": bool, "wait_ticks": int, "demoted": bool}``: the settings above, and whether the library has
+    switched the one-read kernels off on the current GPU because a wait ran into its bound there."""
+    k, v, t, d = C.c_int(0), C.c_int(0), C.c_int64(0), C.c_int(0)
+    _capi.check(_capi.load().ksana_sage_one_read_state(C.byref(k), C.byref(v), C.byref(t), C.byref(d)),
+                "ksana_sage_one_read_state")
+    return {"k": bool(k.value), "v": bool(v.value), "wait_ticks": t.value, "demoted": bool(d.value)}
+
+
+_demotion_logged = False
+
+
+def _log_demotion_once() -> None:
+    """Debug aid of the op path: say once that the library fell back to its two-pass quantizers on this GPU."""
+    global _demotion_logged
+    if _demotion_logged or not log.isEnabledFor(10):  # logging.DEBUG
+        return
+    if one_read_state()["demoted"]:
+        _demotion_logged = True
+        log.debug("Sage HIP path: a one-read quantizer workgroup waited longer than %d ticks for its head on this GPU "
+                  "(the GPU is probably shared); the two-pass quantizers are used from now on (same bits, about "
+                  "15 %% slower) until sage_ops.configure() is called", one_read_state()["wait_ticks"])
+
+
 def _k_lens_arg(k_lens, batch: int, device: torch.device, name: str = "k_lens"):
     """``k_lens`` / ``q_lens`` as the int32 device array the library reads (kept alive by the caller's reference)."""
     if k_lens is None:
@@ -549,6 +583,7 @@ def sageattn(
     ws = workspace_for(q, k) if workspace is None else workspace
     ws.require(q.device, B=B, Hq=Hq, Hkv=k.shape[2], Lq=Lq, Lk=k.shape[1], D=D)
     lib = _capi.load()
+    _log_demotion_once()
     kl = _k_lens_arg(k_lens, B, q.device)
     flags = (_capi.FLAG_PWL_EXP2 if pwl_exp2 else 0) | (_capi.FLAG_SMOOTH_V if smooth_v else 0)
     if prep is not None:

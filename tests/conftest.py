@@ -19,3 +19,14 @@ def hip_device():
     if not torch.cuda.is_available():
         pytest.fail("a test marked gpu ran without a HIP device")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def quant_settings():
+    """``sage_ops.configure`` for one test: the process-wide settings of the one-read quantizers are put back (and the
+    one-read kernels re-armed) when the test ends."""
+    from ksanadit_amd import sage_ops
+
+    before = sage_ops.one_read_state()
+    yield sage_ops.configure
+    sage_ops.configure(one_read=("k" if before["k"] else "") + ("v" if before["v"] else ""), wait_ticks=before["wait_ticks"])

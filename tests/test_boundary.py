@@ -335,3 +335,33 @@ def test_prep_operands_are_converted_once_per_source_tensor():
     table = torch.polar(torch.ones(8, 64), torch.randn(8, 64))  # complex64
     t128 = sage_ops._prep_operand(table, "cpu", torch.complex128)
     assert t128.dtype == torch.complex128 and sage_ops._prep_operand(table, "cpu", torch.complex128) is t128
+
+
+def test_one_read_settings_and_the_occupancy_cache_without_gpu():
+    """``ksana_sage_configure`` validates and stores its settings without touching a device; the launchers' cache of
+    resident-workgroup counts keeps one entry per kernel instantiation (two instantiations of one template have the same
+    function-pointer type, so the type cannot be the key)."""
+    lib = _capi.load()
+    assert lib.ksana_sage_selftest() == 0, lib.ksana_sage_last_error()
+    before = sage_ops.one_read_state()
+    try:
+        assert lib.ksana_sage_configure(b"kx", _capi.KEEP) == _capi.EINVAL and b"letters k and v" in lib.ksana_sage_last_error()
+        sage_ops.configure(one_read="k", wait_ticks=-1)
+        assert sage_ops.one_read_state() == {"k": True, "v": False, "wait_ticks": -1, "demoted": False}
+        sage_ops.configure(one_read="")
+        assert sage_ops.one_read_state() == {"k": False, "v": False, "wait_ticks": -1, "demoted": False}
+        sage_ops.configure(wait_ticks=123)
+        assert sage_ops.one_read_state()["wait_ticks"] == 123 and not sage_ops.one_read_state()["k"]
+    finally:
+        sage_ops.configure(one_read=("k" if before["k"] else "") + ("v" if before["v"] else ""), wait_ticks=before["wait_ticks"])
+    assert sage_ops.one_read_state() == before
+
+
+def test_the_documented_binding_checks_the_current_abi():
+    """INTEGRATION.md's reference-side stub switches itself off when the library's ABI number differs from the one it
+    was written against: that number must be the header's."""
+    root = Path(__file__).resolve().parent.parent
+    header = (root / "include" / "ksana_sage_hip.h").read_text()
+    abi = int(re.search(r"#define KSANA_SAGE_ABI_VERSION (\d+)", header).group(1))
+    doc = (root / "INTEGRATION.md").read_text()
+    assert int(re.search(r"_KSANA_SAGE_ABI = (\d+)", doc).group(1)) == abi == _capi.ABI_VERSION

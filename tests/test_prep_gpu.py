@@ -29,9 +29,9 @@ def _check_q(ws, ref4d, sm_scale, Lq):
 
 def _check_k(ws, ref4d, Lk):
     k_i8, k_scale, k_mean = qr.quant_k_ref(ref4d)
-    assert torch.equal(ws.k_mean.cpu(), k_mean)
-    assert torch.equal(ws.k_scale.cpu(), k_scale)
-    assert torch.equal(untile_k(ws.k_tiles.cpu(), Lk), k_i8)
+    assert torch.equal(ws.k_mean.cpu(), k_mean), "k_mean differs"
+    assert torch.equal(ws.k_scale.cpu(), k_scale), "k_scale differs"
+    assert torch.equal(untile_k(ws.k_tiles.cpu(), Lk), k_i8), "k_int8 differs"
 
 
 @pytest.mark.parametrize(
@@ -70,10 +70,11 @@ def test_quantizer_with_prep_is_bit_exact(hip_device, B, L, H, grids, dtype, nor
 
 
 @pytest.mark.parametrize("kind", ["wan", "qwen"])
-def test_prep_k_stays_exact_when_a_wait_runs_out(hip_device, kind, monkeypatch):
+def test_prep_k_stays_exact_when_a_wait_runs_out(hip_device, kind, quant_settings):
     """K with the norm / rotation step folded in always takes the one-read kernel; a workgroup whose bounded wait
-    runs out recomputes the head's mean from the input, norm and rotation included, in the specified order."""
-    monkeypatch.setenv("KSANA_SAGE_WAIT_TICKS", "0")
+    runs out recomputes the head's mean from the input, norm and rotation included, in the specified order.  A
+    negative bound sends every workgroup but a head's last arriver down that path whatever the timing."""
+    quant_settings(wait_ticks=-1)
     if kind == "wan":
         B, L, H, grids = 1, 1500, 4, [(5, 10, 30)]
         kp, wk = _proj(B, L, H, seed=5)
@@ -96,8 +97,9 @@ def test_prep_k_stays_exact_when_a_wait_runs_out(hip_device, kind, monkeypatch):
     ws.blob.fill_(0x7F)
     sage_ops.quant_k(k4, ws, prep=prep)
     torch.cuda.synchronize()
-    assert sage_ops.quant_status(ws)[0] == 1
+    assert sage_ops.quant_status(ws)[0] == 1, "no workgroup took the recompute path"
     _check_k(ws, k_ref, L)
+    assert not sage_ops.one_read_state()["demoted"], "a test-mode bound must not switch the one-read kernels off"
 
 
 @pytest.mark.parametrize("Lq,Lk,Hq,Hkv,grids", [(300, 300, 12, 12, [(3, 9, 11)]), (200, 520, 4, 4, None), (520, 70, 8, 4, None),

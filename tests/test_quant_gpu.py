@@ -20,12 +20,18 @@ def _run_quant(q, k, v, dev, sm_scale=None, smooth_k=True, expect_status=(0, 0))
     sage_ops.quant_k(kd, ws, smooth_k)
     sage_ops.quant_v(vd, ws)
     torch.cuda.synchronize()
-    assert sage_ops.quant_status(ws) == expect_status, "a quantizer workgroup gave up waiting for its head (or did not, where the test makes it)"
+    if expect_status is not None:
+        assert sage_ops.quant_status(ws) == expect_status, "a quantizer workgroup gave up waiting for its head (or did not, where the test makes it)"
     return ws
 
 
 def _check_against_oracle(q, k, v, dev, sm_scale=None, smooth_k=True, expect_status=(0, 0)):
     ws = _run_quant(q, k, v, dev, sm_scale, smooth_k, expect_status)
+    _compare_with_oracle(ws, q, k, v, sm_scale, smooth_k)
+    return ws
+
+
+def _compare_with_oracle(ws, q, k, v, sm_scale=None, smooth_k=True):
     Lq, Lk = q.shape[1], k.shape[1]
     sm = q.shape[-1] ** -0.5 if sm_scale is None else sm_scale
     qi, qs = qr.quant_q_ref(q, sm)
@@ -197,13 +203,33 @@ def test_v_smoothing_bit_exact(hip_device, B, L, H, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_one_read_kernels_stay_exact_when_a_wait_runs_out(hip_device, dtype, monkeypatch):
-    """The one-read kernels wait, bounded, for the last workgroup of their head.  With the bound set to nothing
-    every workgroup that has to wait gives up at once, flags it, and takes the head's statistic from the input
-    itself: the same bits as ever (the status words say that it happened)."""
-    monkeypatch.setenv("KSANA_SAGE_ONE_READ", "kv")
-    monkeypatch.setenv("KSANA_SAGE_WAIT_TICKS", "0")
+def test_one_read_kernels_stay_exact_when_a_wait_runs_out(hip_device, dtype, quant_settings):
+    """The one-read kernels wait, bounded, for the last workgroup of their head.  With a negative bound every
+    workgroup but a head's last arriver skips the wait, flags it, and takes the head's statistic from the input
+    itself, whatever the timing: the same bits as ever (the status words say that it happened)."""
+    quant_settings(one_read="kv", wait_ticks=-1)
     q, k, v = _rand_qkv(2, 300, 3000, 4, 2, seed=91, dtype=dtype)  # 12 chunks per head, the last one ragged
     _check_against_oracle(q, k, v, hip_device, expect_status=(1, 1))
-    monkeypatch.delenv("KSANA_SAGE_WAIT_TICKS")
+    quant_settings(wait_ticks=0)  # give up at the first poll that finds the flag down: which workgroups do depends on timing
+    ws = _run_quant(q, k, v, hip_device, expect_status=None)
+    _compare_with_oracle(ws, q, k, v)
+    assert not sage_ops.one_read_state()["demoted"]  # test-mode bounds switch nothing off
+    quant_settings(wait_ticks=200000)
     _check_against_oracle(q, k, v, hip_device)  # and the next call on a fresh workspace reports nothing
+
+
+def test_an_expired_production_bound_switches_the_one_read_kernels_off(hip_device, quant_settings):
+    """A positive bound that expires is reported through a word of host memory; from the next call on the library
+    takes the two-pass kernels on this GPU (same bits), until ``configure`` re-arms it."""
+    quant_settings(one_read="kv", wait_ticks=1)  # 10 ns: any workgroup that finds its head's flag down twice gives up
+    q, k, v = _rand_qkv(1, 200, 4000, 4, 4, seed=92)
+    ws = _run_quant(q, k, v, hip_device, expect_status=None)
+    _compare_with_oracle(ws, q, k, v)
+    if sage_ops.quant_status(ws) == (0, 0):
+        pytest.skip("no workgroup had to wait for its head in this run")
+    assert sage_ops.one_read_state()["demoted"]
+    ws = _run_quant(q, k, v, hip_device, expect_status=(0, 0))  # the two-pass kernels: nothing to wait for
+    _compare_with_oracle(ws, q, k, v)
+    quant_settings(wait_ticks=200000)
+    assert not sage_ops.one_read_state()["demoted"]
+    _check_against_oracle(q, k, v, hip_device)

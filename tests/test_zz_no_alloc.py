@@ -68,6 +68,35 @@ def test_static_scratch_entry_point_matches_the_workspace_one(hip_device):
         assert torch.equal(getattr(ws_a, name), getattr(ws_b, name)), name
 
 
+@pytest.mark.gpu
+def test_static_scratch_entry_point_with_the_one_read_kernel(hip_device, quant_settings):
+    """With K set to its one-read kernel the workgroups of a head meet through counters that live in the library's
+    own array too (behind the chunk sums); the bits are those of the workspace variant, the caller's counters are
+    not touched, and a second, smaller call finds the counters cleared."""
+    quant_settings(one_read="kv")
+    dev = hip_device
+    for case, (B, L, H, seed) in enumerate([(2, 2000, 4, 21), (1, 700, 2, 22)]):
+        print(f"one-read call {case}: B={B} L={L} H={H}", flush=True)
+        k = _rand_k(B, L, H, seed)
+        kd = k.to(dev)
+        ws_a = sage_ops.SageWorkspace.allocate(B, H, H, L, L, 128, dev)
+        ws_b = sage_ops.SageWorkspace.allocate(B, H, H, L, L, 128, dev)
+        ws_a.blob.fill_(0xA5)
+        ws_b.blob.fill_(0x5A)
+        sync_before = ws_b.blob[ws_b.layout.k_sync : ws_b.layout.v_sync].clone()
+        _quant_k("ksana_sage_quant_k", kd, ws_a)
+        _quant_k("ksana_sage_quant_k_static", kd, ws_b)
+        torch.cuda.synchronize()
+        assert sage_ops.quant_status(ws_a)[0] == 0
+        for name in ("k_tiles", "k_scale", "k_mean"):
+            assert torch.equal(getattr(ws_a, name), getattr(ws_b, name)), f"call {case}: {name} differs"
+        assert torch.equal(ws_b.blob[ws_b.layout.k_sync : ws_b.layout.v_sync], sync_before)
+        ki, ks, km = qr.quant_k_ref(k, smooth_k=True)
+        assert torch.equal(untile_k(ws_b.k_tiles.cpu(), L), ki)
+        assert torch.equal(ws_b.k_scale.cpu(), ks)
+        assert torch.equal(ws_b.k_mean.cpu(), km.float())
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit():
     """16384 chunk sums is the limit; the refusal comes before any device is touched, so it runs without one."""
     lib = _capi.load()
