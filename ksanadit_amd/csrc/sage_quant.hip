@@ -93,6 +93,22 @@ __device__ __forceinline__ float through_half(float x) {
   return (float)(_Float16)x;
 }
 
+// Two values at a time: one packed conversion instead of two (bf16), the same roundings.
+template <int DT>
+__device__ __forceinline__ void through_half2(float& a, float& b) {
+  asm volatile("" : "+v"(a), "+v"(b));  // as in through_half: the fp32 values exist before they are narrowed
+  if constexpr (DT == KSANA_SAGE_BF16) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    const b2 p = {(__bf16)a, (__bf16)b};
+    const uint32_t w = __builtin_bit_cast(uint32_t, p);
+    a = __uint_as_float(w << 16);
+    b = __uint_as_float(w & 0xffff0000u);
+  } else {
+    a = (float)(_Float16)a;
+    b = (float)(_Float16)b;
+  }
+}
+
 // Rotation factors for the rows of one workgroup, copied to LDS once.  The model's table is
 // [position on an axis][64 pairs] of complex128; a lane needs 8 of them (128 bytes) per row, four
 // times its payload, and fetched straight from the table those reads are 16 bytes out of 30-odd
@@ -182,10 +198,12 @@ __device__ __forceinline__ void prep16_qwen(float* x, const PrepParams& pp, int 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float4 wj = w4[j];
-      x[4 * j + 0] = through_half<DT>((x[4 * j + 0] * r) * wj.x);
-      x[4 * j + 1] = through_half<DT>((x[4 * j + 1] * r) * wj.y);
-      x[4 * j + 2] = through_half<DT>((x[4 * j + 2] * r) * wj.z);
-      x[4 * j + 3] = through_half<DT>((x[4 * j + 3] * r) * wj.w);
+      x[4 * j + 0] = (x[4 * j + 0] * r) * wj.x;
+      x[4 * j + 1] = (x[4 * j + 1] * r) * wj.y;
+      x[4 * j + 2] = (x[4 * j + 2] * r) * wj.z;
+      x[4 * j + 3] = (x[4 * j + 3] * r) * wj.w;
+      through_half2<DT>(x[4 * j + 0], x[4 * j + 1]);
+      through_half2<DT>(x[4 * j + 2], x[4 * j + 3]);
     }
   }
   const float2* tab = txt ? pp.freqs_txt : pp.freqs_img;
@@ -195,12 +213,66 @@ __device__ __forceinline__ void prep16_qwen(float* x, const PrepParams& pp, int 
     for (int j = 0; j < 4; ++j) {
       const float4 cs = t4[j];  // two factors: (re, im), (re, im)
       const float a0 = x[4 * j], b0 = x[4 * j + 1], a1 = x[4 * j + 2], b1 = x[4 * j + 3];
-      x[4 * j + 0] = through_half<DT>(a0 * cs.x - b0 * cs.y);
-      x[4 * j + 1] = through_half<DT>(a0 * cs.y + b0 * cs.x);
-      x[4 * j + 2] = through_half<DT>(a1 * cs.z - b1 * cs.w);
-      x[4 * j + 3] = through_half<DT>(a1 * cs.w + b1 * cs.z);
+      x[4 * j + 0] = a0 * cs.x - b0 * cs.y;
+      x[4 * j + 1] = a0 * cs.y + b0 * cs.x;
+      x[4 * j + 2] = a1 * cs.z - b1 * cs.w;
+      x[4 * j + 3] = a1 * cs.w + b1 * cs.z;
+      through_half2<DT>(x[4 * j + 0], x[4 * j + 1]);
+      through_half2<DT>(x[4 * j + 2], x[4 * j + 3]);
     }
   }
+}
+
+// The pieces of the Wan step on the 16 channels of a lane.
+//   norm16:   y = half( (x * r) * weight[ch] ), r the row's 1 / sqrt(mean(x^2) + eps)
+template <int DT>
+__device__ __forceinline__ void norm16(float* x, float r, const float* w16) {
+  const float4* w4 = reinterpret_cast<const float4*>(w16);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float4 w = w4[j];
+    x[4 * j + 0] = (x[4 * j + 0] * r) * w.x;
+    x[4 * j + 1] = (x[4 * j + 1] * r) * w.y;
+    x[4 * j + 2] = (x[4 * j + 2] * r) * w.z;
+    x[4 * j + 3] = (x[4 * j + 3] * r) * w.w;
+    through_half2<DT>(x[4 * j + 0], x[4 * j + 1]);
+    through_half2<DT>(x[4 * j + 2], x[4 * j + 3]);
+  }
+}
+//   rotate_pair: (a, b) -> half( float( (a + i b) * (c + i s) ) ) in fp64, unfused
+template <int DT>
+__device__ __forceinline__ void rotate_pair(float& xa, float& xb, const double2 cs) {
+  const double a = (double)xa, bb = (double)xb;
+  const double re = a * cs.x - bb * cs.y;
+  const double im = a * cs.y + bb * cs.x;
+  xa = (float)re;
+  xb = (float)im;
+  through_half2<DT>(xa, xb);
+}
+//   comfy_pair: apply_comfyui_rope (utils/rope.py:180-212): out[2i+e] = m[e][0] * x[2i] + m[e][1] * x[2i+1] in fp32, the
+//   first product rounded on its own, the second fused into the sum (what torch's mul followed by addcmul_ computes)
+template <int DT>
+__device__ __forceinline__ void comfy_pair(float& xa, float& xb, const float4 m) {
+  const float a = xa, bb = xb;
+  xa = __fmaf_rn(m.y, bb, __fmul_rn(m.x, a));
+  xb = __fmaf_rn(m.w, bb, __fmul_rn(m.z, a));
+  through_half2<DT>(xa, xb);
+}
+
+// Where the 8 rotation factors of lane c16 (pairs 8 * c16 + j) sit for a token at (frame f, image row hi, column wi):
+// two of the table's three segments at most, the second from pair `split` on.  first / second are element indices of
+// pair 8 * c16 + 0 as if the whole lane lay in that segment (the table is [position][64 pairs]).
+struct RopeLaneIndex {
+  int first, second, split;
+};
+__device__ __forceinline__ RopeLaneIndex rope_lane_index(int c16, int base_f, int base_h, int base_w) {
+  const int i0 = c16 * 8, i7 = c16 * 8 + 7;
+  RopeLaneIndex r;
+  r.first = (i0 < kRopeSplit0 ? base_f : (i0 < kRopeSplit1 ? base_h : base_w)) + i0;
+  r.second = (i7 < kRopeSplit0 ? base_f : (i7 < kRopeSplit1 ? base_h : base_w)) + i0;
+  // pairs [0, 22) frame, [22, 43) image row, [43, 64) column: lane 2 changes segment at pair 22, lane 5 at pair 43
+  r.split = c16 == 2 ? kRopeSplit0 - 16 : (c16 == 5 ? kRopeSplit1 - 40 : 8);
+  return r;
 }
 
 // KIND: PrepParams::kind, a template argument so that every kernel instantiation carries the registers of its own
@@ -215,28 +287,13 @@ __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const Rop
   if (pp.inv_rms != nullptr) {
     // (row_rms: the row's statistic where the caller holds it already, e.g. in LDS)
     const float r = row_rms != nullptr ? *row_rms : pp.inv_rms[(int64_t)b * pp.L + row];
-    const float4* w4 = reinterpret_cast<const float4*>(pp.weight + h * kD + c16 * 16);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float4 w = w4[j];
-      x[4 * j + 0] = through_half<DT>((x[4 * j + 0] * r) * w.x);
-      x[4 * j + 1] = through_half<DT>((x[4 * j + 1] * r) * w.y);
-      x[4 * j + 2] = through_half<DT>((x[4 * j + 2] * r) * w.z);
-      x[4 * j + 3] = through_half<DT>((x[4 * j + 3] * r) * w.w);
-    }
+    norm16<DT>(x, r, pp.weight + h * kD + c16 * 16);
   }
   if constexpr (KIND == 3) {
-    // apply_comfyui_rope (utils/rope.py:180-212): out[2i+e] = m[e][0] * x[2i] + m[e][1] * x[2i+1] in fp32, the first
-    // product rounded on its own, the second fused into the sum (what torch's mul followed by addcmul_ computes)
     if (pp.rot != nullptr && row < pp.rot_rows) {
       const float4* m4 = pp.rot + (int64_t)row * (kD / 2) + c16 * 8;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float4 m = m4[j];
-        const float a = x[2 * j], bb = x[2 * j + 1];
-        x[2 * j] = through_half<DT>(__fmaf_rn(m.y, bb, __fmul_rn(m.x, a)));
-        x[2 * j + 1] = through_half<DT>(__fmaf_rn(m.w, bb, __fmul_rn(m.z, a)));
-      }
+      for (int j = 0; j < 8; ++j) comfy_pair<DT>(x[2 * j], x[2 * j + 1], m4[j]);
     }
     return;
   }
@@ -247,20 +304,11 @@ __device__ __forceinline__ void prep16(float* x, const PrepParams& pp, const Rop
       int rem, wi;
       const int f = small_div(row, plane, &rem);
       const int hi = small_div(rem, gw, &wi);
-      // one table, three segments: the index is picked with integer selects so that every pair is a single
-      // load (selecting between three loads instead makes the compiler branch per pair)
+      // one table, three segments; a lane's 8 pairs lie in two of them at most
       auto rotate = [&](const double2* tab, int base_f, int base_h, int base_w) {
+        const RopeLaneIndex li = rope_lane_index(c16, base_f, base_h, base_w);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int i = c16 * 8 + j;
-          const int idx = (i < kRopeSplit0 ? base_f : (i < kRopeSplit1 ? base_h : base_w)) + i;
-          const double2 cs = tab[idx];
-          const double a = (double)x[2 * j], bb = (double)x[2 * j + 1];
-          const double re = a * cs.x - bb * cs.y;
-          const double im = a * cs.y + bb * cs.x;
-          x[2 * j] = through_half<DT>((float)re);
-          x[2 * j + 1] = through_half<DT>((float)im);
-        }
+        for (int j = 0; j < 8; ++j) rotate_pair<DT>(x[2 * j], x[2 * j + 1], tab[(j < li.split ? li.first : li.second) + j]);
       };
       if (pp.lds_frames > 0 && staged)  // uniform (staged == false: a row outside the rows `rl` was staged for)
         rotate(rl.frame, (f - rl.f0) * kRopeN0,
@@ -502,21 +550,73 @@ __device__ __forceinline__ float lane_xor(float v) {
   return __int_as_float(__builtin_amdgcn_mov_dpp(t, 0x1B, 0xF, 0xF, true));
 }
 
+// One butterfly stage across lanes c16 and c16 ^ M: every lane takes `own + sign * other` with sign = -1 on the lane
+// that holds the "b" half of a pair.  That lane ought to take `other - own`: it ends up with the negative of its
+// value, exactly (a sum and its mirror image round alike).  Both lanes of any LATER stage's pair agree in bit M of
+// c16, so they carry the same factor and the later butterfly is the mirror image of the right one as a whole: after
+// the three stages a lane holds its transform times (-1)^popcount(c16), which the caller folds into the factor it
+// multiplies with next (fwht_lane_sign).  Written this way the stage is one multiply-add per value whose first
+// operand arrives through DPP - no separate sign flip, and no register written just ahead of the DPP read.
+// The instruction is written out: the compiler keeps the DPP move and the multiply-add apart (two instructions per
+// value).  Eight values per statement; `s_nop 1` in front gives the two wait states a DPP read needs after a
+// vector-ALU write of the same register, whatever instruction the compiler placed just before; inside a statement
+// every register is read at least eight instructions after it was written.
+#define KSANA_FMAC_DPP8(CTRL)                                                                                      \
+  "v_fmac_f32_dpp %0, %0, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %1, %1, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %2, %2, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %3, %3, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %4, %4, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %5, %5, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %6, %6, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"                                 \
+  "v_fmac_f32_dpp %7, %7, %8 " CTRL " row_mask:0xf bank_mask:0xf bound_ctrl:1"
 template <int M>
 __device__ __forceinline__ void fwht_cross_stage(float* x, int c16) {
-  // the lane holding the "b" half of a pair computes a - b as (+a) + (-b)
-  const unsigned flip = (c16 & M) ? 0x80000000u : 0u;
+  const float sign = (c16 & M) ? -1.0f : 1.0f;
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const float other = lane_xor<M>(x[e]);
-    const float own = __uint_as_float(__float_as_uint(x[e]) ^ flip);
-    x[e] = other + own;
+  for (int g = 0; g < 2; ++g) {
+    float* y = x + 8 * g;
+    if constexpr (M == 1) {
+      asm volatile("s_nop 1\n\t" KSANA_FMAC_DPP8("quad_perm:[1,0,3,2]")
+                   : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]), "+v"(y[4]), "+v"(y[5]), "+v"(y[6]), "+v"(y[7])
+                   : "v"(sign));
+    } else if constexpr (M == 2) {
+      asm volatile("s_nop 1\n\t" KSANA_FMAC_DPP8("quad_perm:[2,3,0,1]")
+                   : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]), "+v"(y[4]), "+v"(y[5]), "+v"(y[6]), "+v"(y[7])
+                   : "v"(sign));
+    } else {
+      // lane ^ 4 within 8 = row_half_mirror (lane -> 7 - lane) followed by quad_perm [3,2,1,0] (lane ^ 3)
+      float t[8];
+      asm volatile("s_nop 1\n\t"
+                   "v_mov_b32_dpp %8, %0 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %9, %1 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %10, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %11, %3 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %12, %4 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %13, %5 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %14, %6 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_mov_b32_dpp %15, %7 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %0, %8, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %1, %9, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %2, %10, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %3, %11, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %4, %12, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %5, %13, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %6, %14, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+                   "v_fmac_f32_dpp %7, %15, %16 quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1"
+                   : "+v"(y[0]), "+v"(y[1]), "+v"(y[2]), "+v"(y[3]), "+v"(y[4]), "+v"(y[5]), "+v"(y[6]), "+v"(y[7]),
+                     "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3]), "=&v"(t[4]), "=&v"(t[5]), "=&v"(t[6]), "=&v"(t[7])
+                   : "v"(sign));
+    }
   }
 }
 
+// The factor fwht128 leaves on the values of lane c16 (see fwht_cross_stage).
+__device__ __forceinline__ float fwht_lane_sign(int c16) { return (__popc(c16 & 7) & 1) ? -1.0f : 1.0f; }
+
 // Unnormalised Walsh-Hadamard transform of one 128-channel row held by 8 adjacent lanes x 16
-// values (channel = 16*c16 + e).  Butterflies (a, b) -> (a + b, a - b) with stride 1, 2, 4, 8
-// inside the lane, then 16, 32, 64 across lanes c16 ^ 1, ^ 2, ^ 4 - in exactly that order.
+// values (channel = 16*c16 + e), TIMES fwht_lane_sign(c16).  Butterflies (a, b) -> (a + b, a - b) with stride 1, 2,
+// 4, 8 inside the lane, then 16, 32, 64 across lanes c16 ^ 1, ^ 2, ^ 4 - in exactly that order.
 __device__ __forceinline__ void fwht128(float* x, int c16) {
 #pragma unroll
   for (int s = 1; s < 16; s <<= 1) {
@@ -579,12 +679,13 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
   constexpr int kRowsPerWg = 128, R = kRowsPerWg / kSlots;
   const int64_t bh = (int64_t)b * H + h;
   const RopeLds rl = maybe_stage_rope<PRE>(pp, b, blk * kRowsPerWg, kRowsPerWg);
+  const float premul_lane = premul * fwht_lane_sign(c16);
   auto finish_row = [&](float* xr, int row) {
     fwht128(xr, c16);
     float amax = 0.0f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      xr[e] = xr[e] * premul;
+      xr[e] = xr[e] * premul_lane;
       amax = fmaxf(amax, fabsf(xr[e]));
     }
     amax = fmaxf(amax, lane_xor<1>(amax));
@@ -694,13 +795,41 @@ __global__ __launch_bounds__(kThreads) void quant_q_rows_kernel(const uint16_t* 
   stats(q, sB, sL, L, H * (kD / 8), (float)(H * kD), rms_out, true);
   if (ks.ptr != nullptr) stats(ks.ptr, ks.sB, ks.sL, ks.L, ks.n8, ks.n_channels, ks.inv_rms, false);
   if (r0 >= lq_pad) return;  // rows that exist only in k
-  const RopeLds rl = maybe_stage_rope<KIND>(pp, b, r0, kRowsQ);
   __syncthreads();
   // ---- the heads, four at a time ------------------------------------------------------------------------------
   const int rloc = slot & (kRowsQ - 1), h0 = slot / kRowsQ;
   const int row = r0 + rloc;
   const bool live = row < L;
+  // A token's rotation is the same for every head: the lane's 8 factors (pairs 8 * c16 + j of its row) are fetched
+  // once, straight from the model's table (1 MiB, cache resident), and stay in registers for the whole head walk.
+  bool rotates = false;
+  double2 cs[KIND == 1 ? 8 : 1];
+  float4 rm[KIND == 3 ? 8 : 1];
+  if constexpr (KIND == 1) {
+    if (pp.freqs != nullptr && live) {
+      const int gh = pp.grid[b][1], gw = pp.grid[b][2], plane = gh * gw;
+      if (row < pp.grid[b][0] * plane) {
+        rotates = true;
+        int rem, wi;
+        const int f = small_div(row, plane, &rem);
+        const int hi = small_div(rem, gw, &wi);
+        const RopeLaneIndex li = rope_lane_index(c16, f * (kD / 2), hi * (kD / 2), wi * (kD / 2));
+        const double2* tab = reinterpret_cast<const double2*>(pp.freqs);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) cs[j] = tab[(j < li.split ? li.first : li.second) + j];
+      }
+    }
+  } else {
+    if (pp.rot != nullptr && live && row < pp.rot_rows) {
+      rotates = true;
+      const float4* m4 = pp.rot + (int64_t)row * (kD / 2) + c16 * 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) rm[j] = m4[j];
+    }
+  }
+  const float rinv = s_rms[rloc];
   const uint16_t* base = q + b * sB + (int64_t)row * sL + c16 * 16;
+  const float premul_lane = premul * fwht_lane_sign(c16);
   uint4 nxt[2];
   fetch_row16(base + (int64_t)h0 * sH, live && h0 < H, nxt);
   for (int h = h0; h < H; h += kHeadsQ) {
@@ -709,12 +838,21 @@ __global__ __launch_bounds__(kThreads) void quant_q_rows_kernel(const uint16_t* 
     float xr[16];
     widen8<DT>(cur0, xr);
     widen8<DT>(cur1, xr + 8);
-    if (live) prep16<DT, KIND>(xr, pp, rl, b, row, h, c16, true, &s_rms[rloc]);
+    if (live) {
+      norm16<DT>(xr, rinv, pp.weight + h * kD + c16 * 16);
+      if (rotates) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if constexpr (KIND == 1) rotate_pair<DT>(xr[2 * j], xr[2 * j + 1], cs[j]);
+          else comfy_pair<DT>(xr[2 * j], xr[2 * j + 1], rm[j]);
+        }
+      }
+    }
     fwht128(xr, c16);
     float amax = 0.0f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      xr[e] = xr[e] * premul;
+      xr[e] = xr[e] * premul_lane;
       amax = fmaxf(amax, fabsf(xr[e]));
     }
     amax = fmaxf(amax, lane_xor<1>(amax));
@@ -775,13 +913,14 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
   amax = block_max(amax, s_red);
   const bool nz = amax > 0.0f;
   const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
+  const float inv_lane = inv * fwht_lane_sign(c16);  // the transform left this lane's values times that sign
   if (t == 0) k_scale[bh * nkb + blk] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
   int8_t* tile = k_tiles + (bh * nkb + blk) * (int64_t)kTileBytes;
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int frag = i * 4 + (c16 >> 1);
     const int lane = (c16 & 1) * 32 + slot;
-    store_out16(tile + (frag * 64 + lane) * 16, pack_int8x16(x[i], inv));
+    store_out16(tile + (frag * 64 + lane) * 16, pack_int8x16(x[i], inv_lane));
   }
 }
 
@@ -1010,32 +1149,30 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
   __shared__ float s_part[kFinStage * kD];
 
   // ---- 1. the chunk, and its column sums in the specified order -------------------------------
+  // every load of the chunk goes out first (the rows stay in registers as 16-bit values until the end anyway): 16 KiB
+  // per wave in flight; with the norm / rotation step each row is then worked on in place as it arrives
   uint4 raw[kChunkRowsPerSlot][2];
   float acc[16];
-  uint4 nxt[2];
-  if constexpr (PRE) fetch_row16(base + (int64_t)(ch * kMeanChunk + slot) * sL, ch * kMeanChunk + slot < L, nxt);
+#pragma unroll
+  for (int i = 0; i < kChunkRowsPerSlot; ++i) {
+    const int row = ch * kMeanChunk + i * kSlots + slot;
+    raw[i][0] = raw[i][1] = make_uint4(0, 0, 0, 0);
+    if (row < L) {
+      raw[i][0] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL);
+      raw[i][1] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL + 8);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < kChunkRowsPerSlot; ++i) {
     const int row = ch * kMeanChunk + i * kSlots + slot;
     float x[16];
+    widen8<DT>(raw[i][0], x);
+    widen8<DT>(raw[i][1], x + 8);
     if constexpr (PRE) {
-      // one row at a time, the next row's loads in flight: see quant_q_kernel
-      const uint4 cur0 = nxt[0], cur1 = nxt[1];
-      if (i + 1 < kChunkRowsPerSlot) fetch_row16(base + (int64_t)(row + kSlots) * sL, row + kSlots < L, nxt);
-      widen8<DT>(cur0, x);
-      widen8<DT>(cur1, x + 8);
       if (row < L) prep16<DT, PRE>(x, pp, rl, b, row, h, c16);
       raw[i][0] = narrow8<DT>(x);
       raw[i][1] = narrow8<DT>(x + 8);
       __builtin_amdgcn_sched_barrier(0);
-    } else {
-      raw[i][0] = raw[i][1] = make_uint4(0, 0, 0, 0);
-      if (row < L) {
-        raw[i][0] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL);
-        raw[i][1] = *reinterpret_cast<const uint4*>(base + (int64_t)row * sL + 8);
-      }
-      widen8<DT>(raw[i][0], x);
-      widen8<DT>(raw[i][1], x + 8);
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = i == 0 ? x[e] : acc[e] + x[e];
@@ -1171,13 +1308,14 @@ __global__ __launch_bounds__(kThreads, PRE == 1 ? 3 : 1) void quant_k_fused_kern
     amax = fmaxf(fmaxf(s_red[tt][0], s_red[tt][1]), fmaxf(s_red[tt][2], s_red[tt][3]));
     const bool nz = amax > 0.0f;
     const float inv = nz ? __fdiv_rn(127.0f, amax) : 0.0f;
+    const float inv_lane = inv * fwht_lane_sign(c16);  // the transform left this lane's values times that sign
     if (t == 0) k_scale[(int64_t)bh * nkb + blk] = nz ? __fdiv_rn(amax, 127.0f) : 0.0f;
     int8_t* tile = k_tiles + ((int64_t)bh * nkb + blk) * (int64_t)kTileBytes;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int frag = i * 4 + (c16 >> 1);
       const int ln = (c16 & 1) * 32 + slot;
-      store_out16(tile + (frag * 64 + ln) * 16, pack_int8x16(x[i], inv));
+      store_out16(tile + (frag * 64 + ln) * 16, pack_int8x16(x[i], inv_lane));
     }
   }
 }
@@ -1532,7 +1670,7 @@ hipError_t launch_quant_q_rows(const InTensor& q, int B, int H, int L, int lq_pa
   const dim3 grid((rows + kRowsQ - 1) / kRowsQ, B), block(kThreads);
   PrepParams pp = prep;
   float* rms_out = const_cast<float*>(pp.inv_rms);  // the caller's statistic area: written here, read by nobody else in this launch
-  const size_t lds = plan_rope_lds(&pp, B, kRowsQ);
+  const size_t lds = 0;  // the rotation factors of a token are held in registers across its heads: nothing is staged
   KSANA_DISPATCH_DT(q.dtype, {
     if (pp.kind == 3)
       quant_q_rows_kernel<DT, 3><<<grid, block, lds, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, lq_pad, premul, eps, q_i8, q_scale, pp, rms_out, ks);
