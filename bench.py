@@ -39,6 +39,7 @@ def parse():
     ap.add_argument("--calib-copy-mib", type=int, default=0, help="also run one plain device copy of this many MiB (reference point for HBM traffic counters)")
     ap.add_argument("--skip-extra", action="store_true", help="leave out the block-sparse and norm+RoPE legs (they run after the timed steps)")
     ap.add_argument("--skip-block-sparse", action="store_true", help="leave out the block-sparse leg only")
+    ap.add_argument("--skip-sla", action="store_true", help="leave out the sparse-linear backend's leg")
     ap.add_argument("--skip-causal", action="store_true", help="leave out the causal leg only (it launches the same kernel instantiation as the block-sparse leg)")
     ap.add_argument("--skip-other-workloads", action="store_true", help="leave out the attention timings at the other measured shapes")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target length of the CPU SDPA sample; 0 skips it")
@@ -367,6 +368,64 @@ def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
     }
 
 
+def sla_leg(sage_ops, w, q, k, v, ws, dev, iters, topk=0.1):
+    """Outside the timed step: the sparse-linear backend at the headline shape, part by part (HIP events): the block
+    map (block averages on HIP, then the reference's GEMM + topk + scatter), the block-sparse attention on that map,
+    the linear branch with the block's linear layer and the final sum folded in (HIP), and - for scale - the same
+    branch as the reference issues it (five torch kernels plus the layer plus the sum)."""
+    from ksanadit_amd.backends import sage_sla
+    from ksanadit_amd.config import KsanaSageSLAConfig
+    from ksanadit_amd import pick_attn_op
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(iters)]
+        for e in ev:
+            e[0].record()
+            fn()
+            e[1].record()
+        torch.cuda.synchronize()
+        return pctl([e[0].elapsed_time(e[1]) for e in ev], 0.5)
+
+    proj = torch.nn.Linear(w.D, w.D, bias=True).to(dev).to(q.dtype)
+    sage_ops.quant_q(q, ws, w.D**-0.5)  # the legs before this one left other operands in the workspace
+    sage_ops.quant_k(k, ws, True)
+    sage_ops.quant_v(v, ws)
+    bm, kept = sage_sla.topk_block_map(q, k, ws.k_mean, topk)
+    out = torch.empty_like(q)
+    map_ms = timed(lambda: sage_sla.topk_block_map(q, k, ws.k_mean, topk))
+    pool_ms = timed(lambda: (sage_ops.block_means(q, 128), sage_ops.block_means(k, 64, centre=ws.k_mean)))
+    attn_ms = timed(lambda: sage_ops.attn_fwd(ws, out, block_mask=bm))
+    with torch.no_grad():
+        lin_ms = timed(lambda: sage_ops.sla_linear(q, k, v, proj.weight, proj.bias, add=out, out=out))
+        qh, kh, vh = (t.transpose(1, 2) for t in (q, k, v))
+
+        def eager():
+            o_l = sage_sla.linear_branch(qh, kh, vh)
+            with torch.amp.autocast("cuda", dtype=q.dtype):
+                o_l = proj(o_l)
+            return (out.transpose(1, 2) + o_l).to(q.dtype).transpose(1, 2)
+
+        eager_ms = timed(eager)
+        op = pick_attn_op(KsanaSageSLAConfig(topk=topk))(num_heads=w.H, head_size=w.D, causal=False)
+        e2e_ms = timed(lambda: op(q, k, v, proj_l=proj))
+    nb = w.elements * 2.0
+    return {
+        "what": "SageSLA backend, topk share %.2f: block map + block-sparse attention + linear branch (layer and sum folded in)" % topk,
+        "kept_key_blocks": f"{kept} of {bm.shape[-1]}",
+        "block_map_ms": round(map_ms, 4),
+        "block_map_pooling_part_ms": round(pool_ms, 4),
+        "sparse_attn_ms": round(attn_ms, 4),
+        "sparse_attn_tflops_on_kept_blocks": round(w.flops * kept / bm.shape[-1] / (attn_ms * 1e-3) / 1e12, 1),
+        "linear_branch_ms": round(lin_ms, 4),
+        "linear_branch_gbs": round(5.0 * nb / (lin_ms * 1e-3) / 1e9, 1),
+        "linear_branch_note": "algorithmic bytes 5 x 2N: q, k, v and the sparse result read once, the sum written once",
+        "linear_branch_torch_ms": round(eager_ms, 4),
+        "op_e2e_ms": round(e2e_ms, 4),
+    }
+
+
 def main() -> int:
     args = parse()
     if args.gpus != 1:
@@ -485,6 +544,8 @@ def main() -> int:
             rec["causal"] = causal_leg(sage_ops, w, ws, out, args.pwl_exp2, max(3, args.steps // 2))
     if grid is not None and w.B == 1:
         rec["prep_quantizer"] = prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, max(3, args.steps // 2))
+    if grid is not None and w.B == 1 and not args.skip_sla:
+        rec["sla"] = sla_leg(sage_ops, w, q, k, v, ws, dev, max(3, args.steps // 2))
     if not args.skip_extra and not args.skip_other_workloads:
         del q, k, v, ws, out
         torch.cuda.empty_cache()

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 17
+#define KSANA_SAGE_ABI_VERSION 18
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -244,6 +244,25 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[
  * Replaces the Triton kernel compress_kernel / mean_pool (sage_sla.py:43-75). */
 int ksana_sage_block_means(const void* x, int dtype, const int64_t strides[4], int B, int H, int L, int rows_per_block,
                            const float* centre, void* out, void* stream);
+
+/* The linear-attention branch of the sparse-linear backend and what the backend does with it, in three kernels over
+ * [B, L, H, D] tensors (D = 128; strides as for q/k/v), with phi = softmax over the channels of a row, rounded to the
+ * tensors' dtype:
+ *     kv = sum_l phi(k_l)^T v_l,  ksum = sum_l phi(k_l)                         (each rounded to the dtype)
+ *     out_l = (phi(q_l) kv) / (1e-5 + phi(q_l) . ksum)                          sage_sla.py:135-139, 273-282
+ *     out_l = out_l W^T + bias      when proj_weight != NULL (fp32 [128][128], (out, in); bias fp32 [128] or NULL):
+ *                                   the block's proj_l layer, sage_sla.py:284-285, folded in as phi(q_l) (kv W^T)
+ *     out_l += add_l                when add != NULL: the sparse branch's result, sage_sla.py:286
+ * k and v are read once, q once; out may alias add.  sla_workspace: ksana_sage_sla_workspace_bytes(B, H, L) bytes of
+ * device memory, 256-byte aligned (partial sums of kv per run of rows, added in a fixed order: repeated calls give
+ * the same bits).  Replaces calc_linear and the two feature maps of the reference (five library kernels over
+ * [B, H, L, D] intermediates there). */
+int ksana_sage_sla_workspace_bytes(int B, int H, int L, uint64_t* bytes);
+int ksana_sage_sla_linear(const void* q, const void* k, const void* v, int dtype, const int64_t q_strides[4],
+                          const int64_t k_strides[4], const int64_t v_strides[4], int B, int H, int L,
+                          const float* proj_weight, const float* proj_bias, const void* add,
+                          const int64_t add_strides[4], void* out, const int64_t out_strides[4], void* sla_workspace,
+                          void* stream);
 
 /* Did a workgroup of the last ksana_sage_quant_k / ksana_sage_quant_v on this workspace give up waiting for the
  * others of its head?  Both quantizers can read their input once: a workgroup keeps its rows in registers while the

@@ -10,11 +10,12 @@ Drop-in for ksana/operations/attention/backends/sage_sla.py:100-292.  Per call (
 2. block-sparse quantized attention over the kept blocks (sage_sla.py:196-271) - this package's masked kernel, which
    takes the int8 map as it is, on the operands quantized once for both steps;
 3. a linear-attention branch on softmax feature maps of q and k, passed through the block's ``proj_l`` layer, added
-   to the sparse result (sage_sla.py:273-287).
+   to the sparse result (sage_sla.py:273-287) - the HIP kernels behind ``ksana_sage_sla_linear``: one pass over k and
+   v, one over q, with ``proj_l`` (when it is a plain ``torch.nn.Linear``) and the final sum folded in.
 
-The product of the block averages, the top-k selection and the linear branch are a handful of dense torch operations
-(library GEMMs, ``topk``, ``softmax``), as they are in the reference.  Which of two key blocks with equal products
-makes the cut is whatever ``torch.topk`` decides, there as here.
+The product of the block averages and the top-k selection are three dense torch operations on ``[B, H, nq, nk]``
+tensors (a library GEMM, ``topk``, ``scatter_``), as they are in the reference.  Which of two key blocks with equal
+products makes the cut is whatever ``torch.topk`` decides, there as here.
 """
 
 from __future__ import annotations
@@ -50,7 +51,8 @@ def topk_block_map(query: torch.Tensor, key: torch.Tensor, k_mean: torch.Tensor,
 
 
 def linear_branch(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
-    """Linear attention on softmax feature maps over the channel axis (sage_sla.py:135-139, 273-282); ``[B, H, L, D]``."""
+    """Linear attention on softmax feature maps over the channel axis (sage_sla.py:135-139, 273-282); ``[B, H, L, D]``.
+    The reference's five library calls as they stand - what ``sage_ops.sla_linear`` replaces; kept for measurements."""
     fq = F.softmax(q, dim=-1).contiguous().to(q.dtype)
     fk = F.softmax(k, dim=-1).contiguous().to(q.dtype)
     kv = fk.transpose(-1, -2) @ v
@@ -105,11 +107,15 @@ class SageSLAAttentionImpl(KsanaAttentionBackendImpl):
         sage_ops.quant_v(value, ws)
         block_map, kept = topk_block_map(query, key, ws.k_mean, self.topk)
         o_sparse = sage_ops.attn_fwd(ws, torch.empty_like(query), block_mask=block_map)
-        q, k, v = (t.transpose(1, 2) for t in (query, key, value))  # [B, H, L, D] views
-        o_linear = linear_branch(q, k, v)
-        with torch.amp.autocast("cuda", dtype=query.dtype):
-            o_linear = proj_l(o_linear)
-        out = (o_sparse.transpose(1, 2) + o_linear).to(dtype).transpose(1, 2)
+        if isinstance(proj_l, torch.nn.Linear) and tuple(proj_l.weight.shape) == (query.shape[-1],) * 2:
+            # the layer and the sum of the two branches ride along in the linear branch's second pass
+            out = sage_ops.sla_linear(query, key, value, proj_l.weight, proj_l.bias, add=o_sparse, out=o_sparse)
+        else:
+            o_linear = sage_ops.sla_linear(query, key, value)
+            with torch.amp.autocast("cuda", dtype=query.dtype):
+                o_linear = proj_l(o_linear)
+            out = o_sparse + o_linear.to(o_sparse.dtype)
+        out = out.to(dtype)
         if return_sparsity:
             return out, kept / block_map.shape[-1]
         return out

@@ -15,7 +15,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_NAME = "libksana_sage_hip.so"
 LIB_PATH = PKG_DIR / LIB_NAME
-SOURCES = ("sage_capi.hip", "sage_quant.hip", "sage_attn.hip", "sage_probe.hip")
+SOURCES = ("sage_capi.hip", "sage_quant.hip", "sage_attn.hip", "sage_sla.hip", "sage_probe.hip")
 
 HIPCC_FLAGS = (
     "--offload-arch=gfx950",

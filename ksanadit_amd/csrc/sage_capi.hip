@@ -533,6 +533,49 @@ int ksana_sage_block_means(const void* x, int dtype, const int64_t st[4], int B,
   return e == hipSuccess ? 0 : hip_fail(e, "block means launch");
 }
 
+static int sla_layout(int B, int H, int L, uint64_t* part, uint64_t* m_frag, uint64_t* ksum, uint64_t* total) {
+  if (B < 1 || H < 1 || L < 1 || B > 65535 || H > 65535) return fail(KSANA_SAGE_EINVAL, "bad extent (B=%d H=%d L=%d)", B, H, L);
+  int runs = 1, rows_per_run = L;
+  ksana_sage::plan_sla_runs(B, H, L, &runs, &rows_per_run);
+  const uint64_t bh = (uint64_t)B * H;
+  uint64_t off = 0;
+  *part = off, off = align256(off + bh * runs * (ksana_sage::kD * ksana_sage::kD + ksana_sage::kD) * 4);
+  *m_frag = off, off = align256(off + bh * ksana_sage::kD * ksana_sage::kD * 2);
+  *ksum = off, off = align256(off + bh * ksana_sage::kD * 4);
+  *total = off;
+  return 0;
+}
+
+int ksana_sage_sla_workspace_bytes(int B, int H, int L, uint64_t* bytes) {
+  if (!bytes) return fail(KSANA_SAGE_EINVAL, "out-pointer is null");
+  uint64_t a, b, c;
+  return sla_layout(B, H, L, &a, &b, &c, bytes);
+}
+
+int ksana_sage_sla_linear(const void* q, const void* k, const void* v, int dtype, const int64_t q_st[4],
+                          const int64_t k_st[4], const int64_t v_st[4], int B, int H, int L, const float* proj_weight,
+                          const float* proj_bias, const void* add, const int64_t add_st[4], void* out,
+                          const int64_t out_st[4], void* sla_workspace, void* stream) {
+  uint64_t o_part, o_frag, o_ksum, total;
+  if (int rc = sla_layout(B, H, L, &o_part, &o_frag, &o_ksum, &total)) return rc;
+  if (int rc = check_tensor("q", q, dtype, q_st, B, L, H)) return rc;
+  if (int rc = check_tensor("k", k, dtype, k_st, B, L, H)) return rc;
+  if (int rc = check_tensor("v", v, dtype, v_st, B, L, H)) return rc;
+  if (int rc = check_tensor("out", out, dtype, out_st, B, L, H)) return rc;
+  if (add != nullptr)
+    if (int rc = check_tensor("add", add, dtype, add_st, B, L, H)) return rc;
+  if (int rc = check_ws(sla_workspace)) return rc;
+  if ((reinterpret_cast<uintptr_t>(proj_weight) | reinterpret_cast<uintptr_t>(proj_bias)) & 15u)
+    return fail(KSANA_SAGE_EINVAL, "projection weight / bias not 16-byte aligned");
+  const ksana_sage::InTensor at = add != nullptr ? in_tensor(add, dtype, add_st) : ksana_sage::InTensor{};
+  const ksana_sage::OutTensor ot{static_cast<uint16_t*>(out), out_st[0], out_st[1], out_st[2], dtype};
+  hipError_t e = ksana_sage::launch_sla_linear(in_tensor(q, dtype, q_st), in_tensor(k, dtype, k_st), in_tensor(v, dtype, v_st), B, H, L,
+                                               proj_weight, proj_bias, add != nullptr ? &at : nullptr, ot,
+                                               ws_at<float>(sla_workspace, o_part), ws_at<uint16_t>(sla_workspace, o_frag),
+                                               ws_at<float>(sla_workspace, o_ksum), static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? 0 : hip_fail(e, "sla linear branch launch");
+}
+
 int ksana_sage_attn_key_split(const ksana_sage_shape* s, int* first_workgroup, int* runs) {
   if (int rc = check_shape(s)) return rc;
   if (!first_workgroup || !runs) return fail(KSANA_SAGE_EINVAL, "out-pointer is null");

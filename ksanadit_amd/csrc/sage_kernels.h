@@ -139,6 +139,15 @@ hipError_t launch_quant_v_fused(const InTensor& v, int B, int H, int L, int nkb,
 hipError_t launch_block_means(const InTensor& x, int B, int H, int L, int rows, const float* centre, uint16_t* out,
                               hipStream_t s);
 
+// The linear-attention branch of the sparse-linear backend (sage_sla.hip).  part: [B * H][runs][128 * 128 + 128] fp32
+// (plan_sla_runs gives runs); m_frag: [B * H][128 * 128] halves; ksum: [B * H][128] fp32.  proj_w: fp32 [128][128]
+// (out, in) or nullptr; proj_b: fp32 [128] or nullptr; add: a [B, L, H, D] tensor added to the result, or nullptr.
+void plan_sla_runs(int B, int H, int L, int* runs, int* rows_per_run);
+struct OutTensor;
+hipError_t launch_sla_linear(const InTensor& q, const InTensor& k, const InTensor& v, int B, int H, int L,
+                             const float* proj_w, const float* proj_b, const InTensor* add, const OutTensor& out,
+                             float* part, uint16_t* m_frag, float* ksum, hipStream_t s);
+
 struct AttnParams {
   const int8_t* q_i8;
   const float* q_scale;

@@ -412,6 +412,53 @@ def block_means(x: torch.Tensor, rows: int, centre: torch.Tensor | None = None) 
     return out
 
 
+def sla_linear(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, proj_weight: torch.Tensor | None = None,
+               proj_bias: torch.Tensor | None = None, add: torch.Tensor | None = None,
+               out: torch.Tensor | None = None) -> torch.Tensor:
+    """The linear-attention branch of the sparse-linear backend on ``[B, L, H, 128]`` tensors (sage_sla.py:135-139,
+    273-287): ``(phi(q) (phi(k)^T v)) / (1e-5 + phi(q) . sum phi(k))`` with ``phi`` = softmax over the channels, then
+    (optionally) the block's linear layer ``proj_weight`` ``[128, 128]`` / ``proj_bias`` ``[128]`` applied to it and
+    ``add`` (same shape as q; the sparse branch's result) added - all inside two passes over the inputs.  Returns
+    ``[B, L, H, 128]`` in q's dtype; ``out`` may be ``add`` itself."""
+    _require_hip(q, k, v)
+    if q.dim() != 4 or q.shape[3] != 128 or k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("sla_linear expects q, k, v of one shape [B, L, H, 128]")
+    q, k, v = _usable(q), _usable(k), _usable(v)
+    B, L, H, D = q.shape
+    if out is None:
+        out = torch.empty((B, L, H, D), dtype=q.dtype, device=q.device)
+    if out.shape != q.shape or out.dtype != q.dtype or out.device != q.device or _usable(out) is not out:
+        raise ValueError("out must have q's shape, dtype and device, with a unit channel stride")
+    if add is not None:
+        if add.shape != q.shape or add.dtype != q.dtype or add.device != q.device:
+            raise ValueError("add must have q's shape, dtype and device")
+        if add is not out:
+            add = _usable(add)
+    w = b = None
+    if proj_weight is not None:
+        if tuple(proj_weight.shape) != (D, D):
+            raise ValueError(f"proj_weight must be [{D}, {D}]")
+        # the layer runs in the tensors' dtype under autocast: the weight is rounded to it first
+        w = _prep_operand(_prep_operand(proj_weight, q.device, q.dtype), q.device, torch.float32)
+        if proj_bias is not None:
+            if proj_bias.numel() != D:
+                raise ValueError(f"proj_bias must hold {D} values")
+            b = _prep_operand(_prep_operand(proj_bias, q.device, q.dtype), q.device, torch.float32)
+    elif proj_bias is not None:
+        raise ValueError("proj_bias given without proj_weight")
+    lib = _capi.load()
+    nbytes = C.c_uint64(0)
+    _capi.check(lib.ksana_sage_sla_workspace_bytes(B, H, L, C.byref(nbytes)), "ksana_sage_sla_workspace_bytes")
+    scratch = torch.empty(nbytes.value, dtype=torch.uint8, device=q.device)
+    rc = lib.ksana_sage_sla_linear(q.data_ptr(), k.data_ptr(), v.data_ptr(), _DTYPES[q.dtype], _strides(q), _strides(k),
+                                   _strides(v), B, H, L, None if w is None else w.data_ptr(),
+                                   None if b is None else b.data_ptr(), None if add is None else add.data_ptr(),
+                                   None if add is None else _strides(add), out.data_ptr(), _strides(out),
+                                   scratch.data_ptr(), _stream_ptr(q.device))
+    _capi.check(rc, "ksana_sage_sla_linear")
+    return out
+
+
 def quant_status(ws: SageWorkspace) -> tuple[int, int]:
     """``(k_status, v_status)`` of the last K / V quantization on ``ws``: 0, or 1 when a workgroup gave up waiting for
     the others of its head and recomputed the head's statistic from the input (same bits, a slow call; see

@@ -431,17 +431,52 @@ def test_sla_backend_sparse_plus_linear(hip_device):
     sage_ops.quant_k(kd, ws, True)
     got_map, got_kept = topk_block_map(qd, kd, ws.k_mean, 0.25)
     assert got_kept == kept and torch.equal(got_map.cpu(), want_map)
-    # the linear branch: the backend's torch composition on the GPU against the oracle's on the CPU
-    lin_gpu = linear_branch(*(t.transpose(1, 2) for t in (qd, kd, vd))).cpu()
+    # the linear branch: the HIP kernels (and the reference's own torch composition on the GPU) against the oracle on the CPU
     lin_ref = linear_branch_ref(q, k, v)
-    assert _cos(lin_gpu, lin_ref) >= 0.9999
-    assert (lin_gpu.float() - lin_ref.float()).abs().max() <= 0.03 * lin_ref.float().abs().max()
+    for name, lin_gpu in (("hip", sage_ops.sla_linear(qd, kd, vd).transpose(1, 2).cpu()),
+                          ("torch", linear_branch(*(t.transpose(1, 2) for t in (qd, kd, vd))).cpu())):
+        assert _cos(lin_gpu, lin_ref) >= 0.9999, name
+        assert (lin_gpu.float() - lin_ref.float()).abs().max() <= 0.03 * lin_ref.float().abs().max(), name
     # the composition: masked SDPA oracle on the oracle's map + the projected oracle branch
     with torch.no_grad():
         lin = proj.cpu().float()(lin_ref.float()).transpose(1, 2)
     ref = sdpa_ref(q, k, v, block_mask=want_map).float() + lin
     assert _cos(out, ref) >= COS_MIN
     assert (out.float() - ref).abs().max() <= 0.1 * max(ref.abs().max().item(), 0.1)
+
+
+@pytest.mark.parametrize("B,L,H,dtype,bias", [(1, 1000, 3, torch.bfloat16, True), (2, 130, 2, torch.float16, False),
+                                              (1, 4100, 40, torch.bfloat16, False)])
+def test_sla_linear_branch_kernels(hip_device, B, L, H, dtype, bias):
+    """``ksana_sage_sla_linear`` (one pass over k and v, one over q) against the oracle's restatement of calc_linear
+    (sage_sla.py:273-282): plain, with the block's linear layer folded in, and with the sparse branch's result added on
+    the way out; ragged lengths, several runs of rows per head, both half types; repeated calls give the same bits."""
+    from oracle.sla_ref import linear_branch_ref
+
+    print(f"case sla linear B={B} L={L} H={H} {dtype} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(L + H)
+    q = (1.5 * torch.randn((B, L, H, 128), generator=g)).to(dtype)
+    k = (1.5 * torch.randn((B, L, H, 128), generator=g) + torch.randn((1, 1, H, 128), generator=g)).to(dtype)
+    v = torch.randn((B, L, H, 128), generator=g).to(dtype)
+    other = torch.randn((B, L, H, 128), generator=g).to(dtype)
+    w = (0.1 * torch.randn((128, 128), generator=g)).to(dtype)
+    bvec = (0.1 * torch.randn(128, generator=g)).to(dtype) if bias else None
+    qd, kd, vd, od = (t.to(hip_device) for t in (q, k, v, other))
+    ref = linear_branch_ref(q, k, v).transpose(1, 2).float()  # [B, L, H, D]
+    scale = ref.abs().max().item()
+    plain = sage_ops.sla_linear(qd, kd, vd)
+    assert torch.equal(plain, sage_ops.sla_linear(qd, kd, vd)), "two calls on the same inputs differ"
+    plain = plain.cpu().float()
+    assert _cos(plain, ref) >= 0.9999 and (plain - ref).abs().max() <= 0.03 * scale
+    # projected and added: the oracle applies the layer to its (rounded) branch, as the reference does
+    proj = ref.to(dtype).float() @ w.float().t() + (bvec.float() if bias else 0.0)
+    want = proj.to(dtype).float() + other.float()
+    got = sage_ops.sla_linear(qd, kd, vd, w.to(hip_device), None if bvec is None else bvec.to(hip_device), add=od).cpu().float()
+    assert _cos(got, want) >= 0.9999
+    assert (got - want).abs().max() <= 0.03 * max(proj.abs().max().item(), 1e-3) + 0.008 * other.abs().max().item()
+    # in place on the tensor that is added
+    same = sage_ops.sla_linear(qd, kd, vd, w.to(hip_device), None if bvec is None else bvec.to(hip_device), add=od, out=od)
+    assert same.data_ptr() == od.data_ptr() and torch.equal(same.cpu().float(), got)
 
 
 def test_forward_replays_from_a_hip_graph(hip_device):
