@@ -212,6 +212,21 @@ def other_workloads(sage_ops, dev, pwl, iters=7):
                        "quantizer_ms": round(ev[0].elapsed_time(ev[1]), 4)}
         del q, k, v, ws, out
         torch.cuda.empty_cache()
+    # Peaked attention, made on purpose: the headline distributions with q scaled by 4 (every score 4 times as far from
+    # its row's mean), with and without the tile skip (KSANA_SAGE_FLAG_TILE_SKIP: same bits, see the header)
+    if not pwl:
+        w = WORKLOADS["wan14b_480p"]
+        q, k, v = device_inputs(w, dev)
+        q = (q.float() * 4.0).to(torch.bfloat16)
+        ws = sage_ops.workspace_for(q, k)
+        out, out2 = torch.empty_like(q), torch.empty_like(q)
+        sage_ops.quant_q(q, ws, w.D**-0.5), sage_ops.quant_k(k, ws, True), sage_ops.quant_v(v, ws)
+        full = pctl(time_attention(sage_ops, ws, out, iters), 0.5)
+        skip = pctl(time_attention(sage_ops, ws, out2, iters, tile_skip=True), 0.5)
+        res["wan14b_480p_scores_x4"] = {"shape": f"B={w.B} H={w.H} L={w.L} D={w.D}, q x 4", "attn_kernel_ms": round(full, 4),
+                                        "attn_kernel_ms_tile_skip": round(skip, 4), "same_bits": bool(torch.equal(out, out2))}
+        del q, k, v, ws, out, out2
+        torch.cuda.empty_cache()
     return res
 
 

@@ -61,6 +61,15 @@ extern "C" {
 #define KSANA_SAGE_BLKQ 1
 #define KSANA_SAGE_BLKK 64
 
+#define KSANA_SAGE_FLAG_TILE_SKIP 16 /* attention entry points (not with KSANA_SAGE_FLAG_PWL_EXP2): a wave leaves out the  */
+                                     /* exponentials and e4m3 conversions of a key tile whose scores lie more than 17     */
+                                     /* octaves below the softmax reference point of each of its 32 rows.  Every          */
+                                     /* probability byte of such a tile is the zero code, so the result is the same bits  */
+                                     /* - the pvthreshold argument of the reference's sparse kernel (sage_sla.py:237-253; */
+                                     /* the reference passes 1e6, i.e. "never"), at a threshold where nothing changes.    */
+                                     /* Off by default: the test per tile costs ~7 % where no tile qualifies (flat         */
+                                     /* attention); it pays where attention is peaked.                                     */
+
 typedef struct ksana_sage_shape {
   int32_t B;   /* batch                                                     */
   int32_t Hq;  /* query heads                                               */

@@ -19,6 +19,7 @@ FLAG_PWL_EXP2 = 1
 FLAG_SMOOTH_V = 2
 FLAG_WG_4_WAVES = 4
 FLAG_WG_8_WAVES = 8
+FLAG_TILE_SKIP = 16
 PREP_WAN, PREP_WAN_COMFY, PREP_QWEN = 0, 1, 2
 KEEP = -(2**63)  # KSANA_SAGE_KEEP
 

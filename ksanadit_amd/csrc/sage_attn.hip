@@ -143,7 +143,7 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
 // kSplit: the workgroup takes one of `p.n_split` equal runs of key tiles of its (head, query block) and leaves
 // unnormalised accumulators, running maxima and row sums in the workspace for sage_attn_merge_kernel.  Used for
 // the workgroups beyond the last full round of the chip, which would otherwise hold it for a whole round alone.
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW>
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW, bool kTileSkip>
 __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg,
                                                                                    int n_wg, int wg_per_xcd) {
   static_assert(!(kSparse && kSplit), "the key split is built for the dense loop only");
@@ -151,6 +151,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   using Shape = WgShape<kW>;
   constexpr int kThreadsAttn = Shape::kThreads, kRowsWg = Shape::kRows, kStages = Shape::kStages, kAhead = Shape::kAhead;
   constexpr int kListMax = kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4;
+  static_assert(!(kTileSkip && kPwlExp), "the piecewise-linear code formula has its own zero point: no tiles are skipped there");
   int wg, split = 0;
   if constexpr (kSplit) {
     const int item = blockIdx.x / p.n_split;
@@ -513,6 +514,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     return max(max(max8(blk[0], 0), max8(blk[0], 8)), max(max8(blk[1], 0), max8(blk[1], 8)));
   };
   // new running max of query l32 given this lane's tile maximum; returns 2^(old max - new max)
+  bool tile_is_nothing = false;  // set by update_max, per lane
   auto update_max = [&](int imax, float sc, float mneg) -> float {
     {
       // the other half of query l32's keys lives in lane l32 + 32
@@ -525,6 +527,10 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     const float m_new = m_tile > m_run + (kPwlExp ? kLazyMaxPwl : kLazyMax) ? m_tile : m_run;  // -inf at the first tile: always taken
     const float alpha = fast_exp2(m_run - m_new);                     // exactly 1 where the reference point stays
     m_run = m_new;
+    // Every probability of this row in this tile is below 2^(m_tile - m_run + shift).  Under 2^-10 (half the smallest
+    // e4m3 subnormal; a tie goes to the even code, zero) each one converts to the zero code - taken with a margin of
+    // one octave for the exponent's few units of rounding.
+    tile_is_nothing = m_tile < m_run - (kPShift + 11.0f);
     return alpha;
   };
   // p = exp2(sc*dot - m_run + shift); the magic is folded into the constant c, which is off by
@@ -611,6 +617,13 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     const float scp = kPwlExp ? 8.0f * sc : sc;
     const float cp = kPwlExp ? __builtin_fmaf(8.0f, c, 55.5f) : c;
     int pm[4];
+    // A tile whose scores lie more than 17 octaves under the reference point of every one of the wave's 32 rows: each
+    // probability byte would be the zero code.  The wave then writes the zeros directly and leaves out the 64
+    // exponentials and 32 conversions per lane (every chunk below tests this one scalar); the matrix work that
+    // concerns the neighbouring tiles stays.  Same bits either way - the pvthreshold idea of the reference's sparse
+    // kernel (sage_sla.py:237-253) with a threshold at which nothing changes.
+    bool nothing = false;  // wave-uniform
+    if constexpr (kTileSkip) nothing = mine && __all(tile_is_nothing);
     // The S^T chunks are short (a 32-cycle MFMA each): a wave inside them goes ahead of the SIMD's other
     // wave, which is usually in its PV chunks and has 64-cycle MFMAs to hide behind (measured: -1.3 %).
     __builtin_amdgcn_s_setprio(1);
@@ -631,7 +644,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
         int wi = (int)w;
         if (i & 1) pin(wi);
         pf[i >> 1] = wi;
-      } else {
+      } else if (!nothing) {
         const float e0 = p_of(s_cur[0][2 * i], scp, cp), e1 = p_of(s_cur[0][2 * i + 1], scp, cp);
         if (i & 1) {
           int w = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, pf[i >> 1], true);
@@ -640,6 +653,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
         } else {
           pf[i >> 1] = __builtin_amdgcn_cvt_pk_fp8_f32(e0, e1, __float_as_int(e0), false);  // both halves get written
         }
+      } else {
+        pf[i >> 1] = 0;
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -653,7 +668,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     for (int dt = 0; dt < 4; ++dt) {
       if (dt == 0) vf[3] = v_frag(3);
       oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
-      int w = pack4(s_cur[1][4 * dt], s_cur[1][4 * dt + 1], s_cur[1][4 * dt + 2], s_cur[1][4 * dt + 3], scp, cp);
+      int w = 0;
+      if (!nothing) w = pack4(s_cur[1][4 * dt], s_cur[1][4 * dt + 1], s_cur[1][4 * dt + 2], s_cur[1][4 * dt + 3], scp, cp);
       pin(w);
       pf[4 + dt] = w;
       pm[dt] = max8(s_nxt[dt >> 1], (dt & 1) * 8);
@@ -848,7 +864,7 @@ constexpr size_t max_lds() {
                  : WgShape<kW>::kRingBytes + 1024 + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
 }
 
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8>
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8, bool kTileSkip = false>
 hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
   // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
@@ -859,19 +875,22 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg,
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   if (!requested[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW>),
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_lds<kSparse, kW>());
     if (e != hipSuccess) return e;
     requested[dev].store(true, std::memory_order_release);
   }
-  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
 }
 
-// the four (dtype, exp2 form) instantiations behind one (mask, split, workgroup shape) choice
+// the (dtype, exp2 form, tile skip) instantiations behind one (mask, split, workgroup shape) choice
 template <bool kSparse, bool kSplit, int kW>
 hipError_t launch_shape(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd, hipStream_t s) {
   const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
+  if (p.exact_exp2 && p.tile_skip)
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   if (p.exact_exp2)
     return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
                 : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);

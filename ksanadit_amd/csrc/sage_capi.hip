@@ -602,8 +602,10 @@ int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_mask(s, block_mask, mask_st)) return rc;
   if (int rc = check_causal(s, causal)) return rc;
-  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_WG_4_WAVES | KSANA_SAGE_FLAG_WG_8_WAVES))
+  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_WG_4_WAVES | KSANA_SAGE_FLAG_WG_8_WAVES | KSANA_SAGE_FLAG_TILE_SKIP))
     return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
+  if ((flags & KSANA_SAGE_FLAG_TILE_SKIP) && (flags & KSANA_SAGE_FLAG_PWL_EXP2))
+    return fail(KSANA_SAGE_EINVAL, "KSANA_SAGE_FLAG_TILE_SKIP goes with the exact exponential only, not with KSANA_SAGE_FLAG_PWL_EXP2");
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
   if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
@@ -633,6 +635,7 @@ int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[
   p.mask_sH = block_mask ? mask_st[1] : 0;
   p.causal = causal ? 1 : 0;
   p.d_out = s->D;
+  p.tile_skip = (flags & KSANA_SAGE_FLAG_TILE_SKIP) ? 1 : 0;
   hipError_t e = ksana_sage::launch_attn_fwd(p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? 0 : hip_fail(e, "attention launch");
 }
@@ -678,7 +681,8 @@ int forward_impl(const void* q, const void* k, const void* v, void* o, int dtype
   if (int rc = check_tensor("v", v, dtype, v_st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_tensor("o", o, dtype, o_st, s->B, s->Lq, s->Hq)) return rc;
   if (int rc = check_ws(ws)) return rc;
-  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_SMOOTH_V | KSANA_SAGE_FLAG_WG_4_WAVES | KSANA_SAGE_FLAG_WG_8_WAVES))
+  if (flags & ~(KSANA_SAGE_FLAG_PWL_EXP2 | KSANA_SAGE_FLAG_SMOOTH_V | KSANA_SAGE_FLAG_WG_4_WAVES | KSANA_SAGE_FLAG_WG_8_WAVES |
+                KSANA_SAGE_FLAG_TILE_SKIP))
     return fail(KSANA_SAGE_EINVAL, "unknown flag bits 0x%x", flags);
   if (reinterpret_cast<uintptr_t>(k_lens) & 3) return fail(KSANA_SAGE_EINVAL, "k_lens is not 4-byte aligned");
   {

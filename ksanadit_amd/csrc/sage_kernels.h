@@ -173,6 +173,8 @@ struct AttnParams {
   int split_first_wg, n_split;  // filled in by the launcher
   int wg_waves;  // 0: the launcher picks the workgroup shape; 4 or 8: forced (for measurements and tests)
   int d_out;     // channels of an output row that exist: 128, or 64 (head size 64 runs zero-padded to 128)
+  int tile_skip; // 1: a wave leaves out the exponentials of a key tile whose probabilities would all be the zero code
+                 // (same bits; pays on peaked attention, costs ~7 % where no tile qualifies); 0: every tile in full
 };
 constexpr int kMaxSplitPartials = 256;  // (workgroups beyond the last full round) x (runs each) never exceeds this
 constexpr int kMinTilesPerSplit = 8;    // a run shorter than this does not repay its prologue

@@ -479,6 +479,37 @@ def test_sla_linear_branch_kernels(hip_device, B, L, H, dtype, bias):
     assert same.data_ptr() == od.data_ptr() and torch.equal(same.cpu().float(), got)
 
 
+@pytest.mark.parametrize("mode", ["dense8", "dense4", "masked", "causal"])
+def test_skipping_tiles_of_zero_probabilities_changes_no_bit(hip_device, mode):
+    """``tile_skip=True``: a wave leaves out the exponentials of a key tile whose probabilities would all convert to the zero e4m3 code
+    (scores more than 17 octaves under every row's reference point).  On peaked scores - queries that lean hard towards
+    one run of keys - many tiles qualify; the output must equal, bit for bit, the one computed with every tile in full."""
+    B, H, L = 1, 2, 2048
+    g = torch.Generator().manual_seed(97)
+    q = torch.randn((B, L, H, 128), generator=g)
+    k = torch.randn((B, L, H, 128), generator=g)
+    v = torch.randn((B, L, H, 128), generator=g)
+    direction = torch.randn(128, generator=g)
+    direction /= direction.norm()
+    q = q + 14.0 * direction                      # every query leans the same way ...
+    k[:, 512:640] += 20.0 * direction             # ... towards these 128 keys: about 35 octaves above the rest
+    k[:, 1500:1510] += 10.0 * direction           # and a few that end up in between, near the threshold
+    qd, kd, vd = (t.to(torch.bfloat16).to(hip_device) for t in (q, k, v))
+    ws = sage_ops.workspace_for(qd, kd)
+    sage_ops.quant_q(qd, ws, 128**-0.5)
+    sage_ops.quant_k(kd, ws, True)
+    sage_ops.quant_v(vd, ws)
+    kwargs = {"dense8": {"wg_waves": 8}, "dense4": {"wg_waves": 4}, "causal": {"causal": True},
+              "masked": {"block_mask": (torch.rand((L // 128, L // 64), generator=g) < 0.7).to(torch.int8)}}[mode]
+    full = sage_ops.attn_fwd(ws, torch.empty_like(qd), **kwargs)
+    skipped = sage_ops.attn_fwd(ws, torch.empty_like(qd), tile_skip=True, **kwargs)
+    torch.cuda.synchronize()
+    assert torch.equal(full, skipped)
+    ref = sdpa_ref(q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16), causal=(mode == "causal"),
+                   block_mask=kwargs.get("block_mask"))
+    assert _cos(skipped.cpu(), ref) >= COS_MIN
+
+
 def test_forward_replays_from_a_hip_graph(hip_device):
     """The C entry points allocate nothing and only launch kernels, so the whole path can be captured once and
     replayed: every replay, with eager work and synchronisation in between, must equal the eager result."""
