@@ -126,7 +126,10 @@ def test_entry_points_validate_before_touching_the_gpu():
     assert lib.ksana_sage_attn_fwd_varlen(fake, fake, _capi.BF16, st, C.byref(shape), null, None, C.c_void_p(0x1002), null,
                                           0, 0, null) == _capi.EINVAL  # q_lens alignment
     assert b"q_lens" in lib.ksana_sage_last_error()
-    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), null, 0, 0x10, null) == _capi.EINVAL  # flags
+    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), null, 0, 0x20, null) == _capi.EINVAL  # flags
+    both = _capi.FLAG_TILE_SKIP | _capi.FLAG_PWL_EXP2  # the skip's zero point is the exact exponential's
+    assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), null, 0, both, null) == _capi.EINVAL
+    assert b"TILE_SKIP" in lib.ksana_sage_last_error()
     assert lib.ksana_sage_attn_fwd(fake, fake, _capi.BF16, st, C.byref(shape), C.c_void_p(0x1002), 0, 0, null) == _capi.EINVAL  # k_lens alignment
     assert lib.ksana_sage_forward(fake, fake, null, fake, _capi.BF16, st, st, st, st, C.byref(shape), null, 0.1, 1, 0, 0, fake, null) == _capi.EINVAL
     # the step-before-attention descriptor is validated on the host as well
