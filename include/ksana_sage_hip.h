@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 18
+#define KSANA_SAGE_ABI_VERSION 19
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -253,6 +253,15 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[
  * Replaces the Triton kernel compress_kernel / mean_pool (sage_sla.py:43-75). */
 int ksana_sage_block_means(const void* x, int dtype, const int64_t strides[4], int B, int H, int L, int rows_per_block,
                            const float* centre, void* out, void* stream);
+
+/* The second half of get_block_map (sage_sla.py:83-90) in one kernel: score = pooled_q pooled_k^T as a tensor of the
+ * blocks' dtype, then per query block ones at the `keep` key blocks with the largest scores (of equal scores the
+ * lower index wins; torch.topk, which the reference calls, leaves that open), zeros elsewhere.  pooled_q / pooled_k:
+ * device, [B, H, nq, 128] / [B, H, nk, 128] in `dtype`, contiguous (what ksana_sage_block_means writes);
+ * block_map: int8 [B, H, nq, nk], contiguous - the mask ksana_sage_attn_fwd_masked takes.  nk <= 1024
+ * (KSANA_SAGE_ENOTSUP beyond).  Replaces a GEMM, torch.topk, zeros_like and scatter_. */
+int ksana_sage_sla_block_map(const void* pooled_q, const void* pooled_k, int dtype, int B, int H, int nq, int nk,
+                             int keep, int8_t* block_map, void* stream);
 
 /* The linear-attention branch of the sparse-linear backend and what the backend does with it, in three kernels over
  * [B, L, H, D] tensors (D = 128; strides as for q/k/v), with phi = softmax over the channels of a row, rounded to the

@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -41,6 +41,7 @@ EXPORTS = (
     "ksana_sage_block_means",
     "ksana_sage_sla_workspace_bytes",
     "ksana_sage_sla_linear",
+    "ksana_sage_sla_block_map",
     "ksana_sage_mfma_probe",
     "ksana_sage_forward",
     "ksana_sage_quant_q_prep",
@@ -122,6 +123,7 @@ def _declare(lib):
     lib.ksana_sage_sla_workspace_bytes.restype = i
     lib.ksana_sage_sla_linear.argtypes = [vp, vp, vp, i, st, st, st, i, i, i, vp, vp, vp, st, vp, st, vp, vp]
     lib.ksana_sage_sla_linear.restype = i
+    lib.ksana_sage_sla_block_map.argtypes, lib.ksana_sage_sla_block_map.restype = [vp, vp, i, i, i, i, i, i, vp, vp], i
     lib.ksana_sage_mfma_probe.argtypes = [vp, C.c_uint64, i, i, vp, C.POINTER(C.c_double)]
     lib.ksana_sage_mfma_probe.restype = i
     lib.ksana_sage_forward.argtypes = [vp, vp, vp, vp, i, st, st, st, st, sp, vp, f, i, i, i, vp, vp]

@@ -13,9 +13,8 @@ Drop-in for ksana/operations/attention/backends/sage_sla.py:100-292.  Per call (
    to the sparse result (sage_sla.py:273-287) - the HIP kernels behind ``ksana_sage_sla_linear``: one pass over k and
    v, one over q, with ``proj_l`` (when it is a plain ``torch.nn.Linear``) and the final sum folded in.
 
-The product of the block averages and the top-k selection are three dense torch operations on ``[B, H, nq, nk]``
-tensors (a library GEMM, ``topk``, ``scatter_``), as they are in the reference.  Which of two key blocks with equal
-products makes the cut is whatever ``torch.topk`` decides, there as here.
+The product of the block averages and the top-k selection are one HIP kernel (``ksana_sage_sla_block_map``; of two key
+blocks with equal products the lower index makes the cut - ``torch.topk``, which the reference calls, leaves that open).
 """
 
 from __future__ import annotations
@@ -31,10 +30,13 @@ from .base import KsanaAttentionBackendImpl
 
 def block_map_from_pooled(pooled_q: torch.Tensor, pooled_k: torch.Tensor, topk_ratio: float) -> tuple[torch.Tensor, int]:
     """int8 ``[B, H, nq, nk]`` with ``topk`` ones per row, and ``topk`` (the second half of ``get_block_map``,
-    sage_sla.py:83-90).  ``pooled_*``: block averages ``[B, H, n, D]``, k's taken after centring."""
-    score = pooled_q @ pooled_k.transpose(-1, -2)
-    nk = score.shape[-1]
+    sage_sla.py:83-90).  ``pooled_*``: block averages ``[B, H, n, D]``, k's taken after centring.  On a HIP device with
+    at most 1024 key blocks this is one kernel (``ksana_sage_sla_block_map``); otherwise the reference's four torch calls."""
+    nk = pooled_k.shape[-2]
     keep = min(nk, int(topk_ratio * nk))
+    if pooled_q.is_cuda and nk <= 1024 and pooled_q.shape[-1] == 128 and pooled_q.dtype in (torch.bfloat16, torch.float16):
+        return sage_ops.sla_block_map(pooled_q, pooled_k, keep), keep
+    score = pooled_q @ pooled_k.transpose(-1, -2)
     picked = torch.topk(score, keep, dim=-1, sorted=False).indices
     block_map = torch.zeros_like(score, dtype=torch.int8)
     block_map.scatter_(-1, picked, 1)

@@ -576,6 +576,19 @@ int ksana_sage_sla_linear(const void* q, const void* k, const void* v, int dtype
   return e == hipSuccess ? 0 : hip_fail(e, "sla linear branch launch");
 }
 
+int ksana_sage_sla_block_map(const void* pooled_q, const void* pooled_k, int dtype, int B, int H, int nq, int nk, int keep,
+                             int8_t* block_map, void* stream) {
+  if (B < 1 || H < 1 || nq < 1 || nk < 1 || (int64_t)B * H > 65535) return fail(KSANA_SAGE_EINVAL, "bad extent (B=%d H=%d nq=%d nk=%d)", B, H, nq, nk);
+  if (dtype != KSANA_SAGE_BF16 && dtype != KSANA_SAGE_FP16) return fail(KSANA_SAGE_EINVAL, "dtype %d unknown", dtype);
+  if (nk > 1024) return fail(KSANA_SAGE_ENOTSUP, "nk=%d key blocks exceed 1024 (a group's scores are kept in LDS)", nk);
+  if (!pooled_q || !pooled_k || !block_map) return fail(KSANA_SAGE_EINVAL, "null pointer");
+  if ((reinterpret_cast<uintptr_t>(pooled_q) | reinterpret_cast<uintptr_t>(pooled_k)) & 15u)
+    return fail(KSANA_SAGE_EINVAL, "pooled blocks not 16-byte aligned");
+  hipError_t e = ksana_sage::launch_sla_block_map(static_cast<const uint16_t*>(pooled_q), static_cast<const uint16_t*>(pooled_k),
+                                                  dtype, B * H, nq, nk, keep, block_map, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? 0 : hip_fail(e, "block map launch");
+}
+
 int ksana_sage_attn_key_split(const ksana_sage_shape* s, int* first_workgroup, int* runs) {
   if (int rc = check_shape(s)) return rc;
   if (!first_workgroup || !runs) return fail(KSANA_SAGE_EINVAL, "out-pointer is null");

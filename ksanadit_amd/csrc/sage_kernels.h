@@ -148,6 +148,11 @@ hipError_t launch_sla_linear(const InTensor& q, const InTensor& k, const InTenso
                              const float* proj_w, const float* proj_b, const InTensor* add, const OutTensor& out,
                              float* part, uint16_t* m_frag, float* ksum, hipStream_t s);
 
+// int8 block_map[BH][nq][nk]: per query block ones at the `keep` key blocks with the largest pooled_q . pooled_k (half
+// tensors [BH][n][128], contiguous); nk <= 1024
+hipError_t launch_sla_block_map(const uint16_t* pooled_q, const uint16_t* pooled_k, int dtype, int BH, int nq, int nk, int keep,
+                                int8_t* block_map, hipStream_t s);
+
 struct AttnParams {
   const int8_t* q_i8;
   const float* q_scale;

@@ -415,6 +415,97 @@ __global__ __launch_bounds__(kSlaThreads, 2) void sla_apply_kernel(const uint16_
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The block map from the pooled blocks (get_block_map, sage_sla.py:83-90): score = pooled_q pooled_k^T as a tensor of
+// the half type (fp32 accumulation, one rounding), then for every query block the `keep` key blocks with the largest
+// scores get a one, the others a zero; of equal scores the lower index wins (what a stable descending sort gives;
+// torch.topk leaves it open).  grid = (ceil(nq / 32), B * H), 256 threads; dynamic LDS 32 * nk_pad * 2 bytes.
+//
+// Scores: 32 query blocks x 32 key blocks per 32x32x16 matrix instruction, contraction over the 128 channels - both
+// operands are 16-byte pieces of pooled rows as they lie in memory; wave w takes the key tiles w, w + 4, ...  Each
+// score goes to LDS as a 16-bit key whose unsigned order is the order of the values.  Selection, one wave per 8 query
+// blocks: the keep-th largest key by bisection over its 16 bits (count of keys >= candidate by ballots), then ones for
+// the keys above it and for as many of its equals, lowest index first, as are still missing.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kMapMaxKeyBlocks = 1024;
+
+template <int DT>
+__global__ __launch_bounds__(kSlaThreads) void sla_block_map_kernel(const uint16_t* __restrict__ pooled_q,
+                                                                    const uint16_t* __restrict__ pooled_k, int nq, int nk,
+                                                                    int nk_pad, int keep, int8_t* __restrict__ block_map) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
+  uint16_t* s_key = reinterpret_cast<uint16_t*>(s_dyn);  // [32][nk_pad]
+  const int bh = blockIdx.y, q0 = blockIdx.x * 32;
+  const int t = threadIdx.x, lane = t & 63;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const uint16_t* pq = pooled_q + ((int64_t)bh * nq + q0 + l32) * kD + 8 * g;
+  const uint16_t* pk = pooled_k + (int64_t)bh * nk * kD + 8 * g;
+  uint4 a[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) a[s] = q0 + l32 < nq ? *reinterpret_cast<const uint4*>(pq + 16 * s) : make_uint4(0, 0, 0, 0);
+  for (int nt = w; nt * 32 < nk_pad; nt += 4) {
+    const int kb = nt * 32 + l32;
+    uint4 b[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) b[s] = kb < nk ? *reinterpret_cast<const uint4*>(pk + (int64_t)kb * kD + 16 * s) : make_uint4(0, 0, 0, 0);
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) acc = mfma32<DT>(a[s], b[s], acc);
+    // register r: query block 8 (r / 4) + 4 g + r % 4 of the group, key block kb
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = 8 * (r >> 2) + 4 * g + (r & 3);
+      uint32_t bits;
+      if constexpr (DT == KSANA_SAGE_BF16)
+        bits = __builtin_bit_cast(uint16_t, (__bf16)acc[r]);
+      else
+        bits = __builtin_bit_cast(uint16_t, (_Float16)acc[r]);
+      const uint32_t key = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);  // unsigned order = value order
+      s_key[m * nk_pad + kb] = (uint16_t)(kb < nk ? key : 0u);                    // padding sorts below everything
+    }
+  }
+  __syncthreads();
+  // a row's keys in registers: lane holds the keys lane + 64 i (0, the padding value, beyond nk)
+  constexpr int kPerLane = kMapMaxKeyBlocks / 64;
+  for (int mi = 0; mi < 8; ++mi) {
+    const int m = 8 * w + mi;
+    if (q0 + m >= nq) break;  // wave-uniform
+    const uint16_t* row = s_key + m * nk_pad;
+    int8_t* out = block_map + ((int64_t)bh * nq + q0 + m) * nk;
+    uint32_t key[kPerLane];
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) key[i] = lane + 64 * i < nk ? row[lane + 64 * i] : 0u;
+    uint32_t thr = 0;
+    if (keep > 0 && keep < nk) {
+      for (int bit = 15; bit >= 0; --bit) {
+        const uint32_t cand = thr | (1u << bit);
+        int count = 0;
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) count += __popcll(__ballot(key[i] >= cand));  // padding keys are 0 < cand
+        if (count >= keep) thr = cand;  // uniform
+      }
+    }
+    int above = 0;
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) above += __popcll(__ballot(key[i] > thr));
+    int missing = keep >= nk ? nk : (keep <= 0 ? 0 : keep - above);  // of the keys equal to thr, lowest index first
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) {
+      const int idx = lane + 64 * i;
+      const bool in = idx < nk;
+      const bool eq = in && key[i] == thr;
+      const unsigned long long bal = __ballot(eq);
+      const int rank = __builtin_amdgcn_mbcnt_hi((unsigned)(bal >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)bal, 0));
+      const bool one = in && keep > 0 && (keep >= nk || key[i] > thr || (eq && rank < missing));
+      if (in) out[idx] = one ? 1 : 0;
+      missing -= __popcll(bal);
+    }
+  }
+}
+
 }  // namespace
 
 // rows per run of sla_kv_partial_kernel: about two workgroups per compute unit in all, runs a multiple of 128 rows
@@ -469,4 +560,19 @@ hipError_t launch_sla_linear(const InTensor& q, const InTensor& k, const InTenso
   return hipGetLastError();
 }
 
+}  // namespace ksana_sage
+
+namespace ksana_sage {
+hipError_t launch_sla_block_map(const uint16_t* pooled_q, const uint16_t* pooled_k, int dtype, int BH, int nq, int nk, int keep,
+                                int8_t* block_map, hipStream_t s) {
+  if (nk > kMapMaxKeyBlocks) return hipErrorInvalidValue;
+  const int nk_pad = (nk + 31) / 32 * 32;
+  const dim3 grid((nq + 31) / 32, BH), block(kSlaThreads);
+  const size_t lds = (size_t)32 * nk_pad * 2;
+  if (dtype == KSANA_SAGE_BF16)
+    sla_block_map_kernel<KSANA_SAGE_BF16><<<grid, block, lds, s>>>(pooled_q, pooled_k, nq, nk, nk_pad, keep, block_map);
+  else
+    sla_block_map_kernel<KSANA_SAGE_FP16><<<grid, block, lds, s>>>(pooled_q, pooled_k, nq, nk, nk_pad, keep, block_map);
+  return hipGetLastError();
+}
 }  // namespace ksana_sage

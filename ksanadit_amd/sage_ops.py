@@ -412,6 +412,24 @@ def block_means(x: torch.Tensor, rows: int, centre: torch.Tensor | None = None) 
     return out
 
 
+def sla_block_map(pooled_q: torch.Tensor, pooled_k: torch.Tensor, keep: int) -> torch.Tensor:
+    """int8 ``[B, H, nq, nk]``: per query block ones at the ``keep`` key blocks with the largest
+    ``pooled_q @ pooled_k^T`` (a tensor of the blocks' dtype); the second half of ``get_block_map`` (sage_sla.py:83-90).
+    ``pooled_*``: ``[B, H, n, 128]`` block averages on a HIP device, at most 1024 key blocks."""
+    _require_hip(pooled_q, pooled_k)
+    if pooled_q.dim() != 4 or pooled_k.dim() != 4 or pooled_q.shape[:2] != pooled_k.shape[:2] or pooled_q.shape[3] != 128 \
+            or pooled_k.shape[3] != 128:
+        raise ValueError("pooled blocks must be [B, H, n, 128] with equal B, H")
+    pooled_q, pooled_k = pooled_q.contiguous(), pooled_k.contiguous()
+    B, H, nq, _ = pooled_q.shape
+    nk = pooled_k.shape[2]
+    block_map = torch.empty((B, H, nq, nk), dtype=torch.int8, device=pooled_q.device)
+    rc = _capi.load().ksana_sage_sla_block_map(pooled_q.data_ptr(), pooled_k.data_ptr(), _DTYPES[pooled_q.dtype], B, H, nq, nk,
+                                               int(keep), block_map.data_ptr(), _stream_ptr(pooled_q.device))
+    _capi.check(rc, "ksana_sage_sla_block_map")
+    return block_map
+
+
 def sla_linear(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, proj_weight: torch.Tensor | None = None,
                proj_bias: torch.Tensor | None = None, add: torch.Tensor | None = None,
                out: torch.Tensor | None = None) -> torch.Tensor:

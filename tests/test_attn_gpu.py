@@ -445,6 +445,27 @@ def test_sla_backend_sparse_plus_linear(hip_device):
     assert (out.float() - ref).abs().max() <= 0.1 * max(ref.abs().max().item(), 0.1)
 
 
+@pytest.mark.parametrize("B,H,nq,nk,keep,dtype", [(1, 2, 45, 70, 9, torch.bfloat16), (2, 3, 8, 512, 51, torch.float16),
+                                                   (1, 1, 33, 1024, 1, torch.bfloat16), (1, 2, 16, 96, 0, torch.bfloat16),
+                                                   (1, 2, 16, 96, 96, torch.bfloat16), (1, 40, 256, 512, 51, torch.bfloat16)])
+def test_block_map_kernel_on_exact_scores_with_ties(hip_device, B, H, nq, nk, keep, dtype):
+    """``ksana_sage_sla_block_map`` (scores + top-k + map in one kernel) on pooled blocks of small integers: every
+    score is exact in the half type, so the expected map is computable exactly - and full of ties, which go to the
+    lower index (a stable descending sort; sage_sla.py:83-90 leaves them to torch.topk)."""
+    print(f"case block map B={B} H={H} nq={nq} nk={nk} keep={keep} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(nq * 7 + nk)
+    pq = torch.randint(-1, 2, (B, H, nq, 128), generator=g).to(dtype)
+    pk = torch.randint(-1, 2, (B, H, nk, 128), generator=g).to(dtype)
+    pk[:, :, nk // 2] = pk[:, :, 0]  # two identical key blocks: an exact tie in every row
+    score = (pq.float() @ pk.float().transpose(-1, -2)).to(dtype).float()
+    order = score.sort(dim=-1, descending=True, stable=True).indices
+    want = torch.zeros((B, H, nq, nk), dtype=torch.int8)
+    want.scatter_(-1, order[..., :keep], 1)
+    got = sage_ops.sla_block_map(pq.to(hip_device), pk.to(hip_device), keep).cpu()
+    assert got.dtype == torch.int8 and torch.equal(got.sum(-1), torch.full((B, H, nq), keep, dtype=got.sum(-1).dtype))
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("B,L,H,dtype,bias", [(1, 1000, 3, torch.bfloat16, True), (2, 130, 2, torch.float16, False),
                                               (1, 4100, 40, torch.bfloat16, False)])
 def test_sla_linear_branch_kernels(hip_device, B, L, H, dtype, bias):
