@@ -2,6 +2,8 @@
 // Declarations and the reference call sites each entry point replaces: include/ksana_sage_hip.h.
 #include <hip/hip_runtime.h>
 
+#include <dlfcn.h>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -35,6 +37,46 @@ int fail(int code, const char* fmt, ...) {
 }
 
 uint64_t align256(uint64_t x) { return (x + 255u) & ~uint64_t(255); }
+
+// Named ranges around the stages of a call (quantize, attention, ...) for a timeline viewer: roctx push / pop, looked
+// up at run time in the profiler's marker library the first time they are wanted - only when the environment variable
+// KSANA_SAGE_ROCTX is set to something other than 0 (read once), so a process that is not being profiled pays one
+// branch per stage and links against nothing.
+class StageRange {
+ public:
+  explicit StageRange(const char* name) : on_(enabled()) {
+    if (on_) push_(name);
+  }
+  ~StageRange() {
+    if (on_) pop_();
+  }
+  StageRange(const StageRange&) = delete;
+  StageRange& operator=(const StageRange&) = delete;
+
+ private:
+  using Push = int (*)(const char*);
+  using Pop = int (*)();
+  static Push push_;
+  static Pop pop_;
+  static bool enabled() {
+    static const bool on = [] {
+      const char* e = getenv("KSANA_SAGE_ROCTX");
+      if (e == nullptr || *e == 0 || strcmp(e, "0") == 0) return false;
+      for (const char* lib : {"librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1", "libroctx64.so", "libroctx64.so.4"}) {
+        if (void* h = dlopen(lib, RTLD_NOW | RTLD_GLOBAL)) {
+          push_ = reinterpret_cast<Push>(dlsym(h, "roctxRangePushA"));
+          pop_ = reinterpret_cast<Pop>(dlsym(h, "roctxRangePop"));
+          if (push_ != nullptr && pop_ != nullptr) return true;
+        }
+      }
+      return false;
+    }();
+    return on;
+  }
+  bool on_;
+};
+StageRange::Push StageRange::push_ = nullptr;
+StageRange::Pop StageRange::pop_ = nullptr;
 
 int check_shape(const ksana_sage_shape* s) {
   if (!s) return fail(KSANA_SAGE_EINVAL, "shape is null");
@@ -316,6 +358,7 @@ int ksana_sage_quant_q(const void* q, int dtype, const int64_t st[4], const ksan
 static int quant_q_impl(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                         const ksana_sage_prep* prep, float sm_scale, void* ws, void* stream, const void* k,
                         const int64_t k_st[4], bool* k_rms_done) {
+  const StageRange range("ksana_sage.quant_q");
   if (k_rms_done) *k_rms_done = false;
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("q", q, dtype, st, s->B, s->Lq, s->Hq)) return rc;
@@ -363,6 +406,7 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
 static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                         const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, int* sync_words,
                         void* stream, bool rms_done = false, bool may_allocate = true) {
+  const StageRange range("ksana_sage.quant_k");
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -458,6 +502,7 @@ int ksana_sage_quant_v(const void* v, int dtype, const int64_t st[4], const ksan
 
 int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_v,
                               void* ws, void* stream) {
+  const StageRange range("ksana_sage.quant_v");
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("v", v, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
   if (int rc = check_ws(ws)) return rc;
@@ -556,6 +601,7 @@ int ksana_sage_sla_linear(const void* q, const void* k, const void* v, int dtype
                           const int64_t k_st[4], const int64_t v_st[4], int B, int H, int L, const float* proj_weight,
                           const float* proj_bias, const void* add, const int64_t add_st[4], void* out,
                           const int64_t out_st[4], void* sla_workspace, void* stream) {
+  const StageRange range("ksana_sage.sla_linear");
   uint64_t o_part, o_frag, o_ksum, total;
   if (int rc = sla_layout(B, H, L, &o_part, &o_frag, &o_ksum, &total)) return rc;
   if (int rc = check_tensor("q", q, dtype, q_st, B, L, H)) return rc;
@@ -612,6 +658,7 @@ int ksana_sage_attn_fwd_masked(void* ws, void* o, int dtype, const int64_t o_st[
 int ksana_sage_attn_fwd_varlen(void* ws, void* o, int dtype, const int64_t o_st[4], const ksana_sage_shape* s,
                                const int8_t* block_mask, const int64_t mask_st[2], const int32_t* q_lens,
                                const int32_t* k_lens, int causal, int flags, void* stream) {
+  const StageRange range("ksana_sage.attention");
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_mask(s, block_mask, mask_st)) return rc;
   if (int rc = check_causal(s, causal)) return rc;

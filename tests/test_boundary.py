@@ -368,3 +368,19 @@ def test_the_documented_binding_checks_the_current_abi():
     abi = int(re.search(r"#define KSANA_SAGE_ABI_VERSION (\d+)", header).group(1))
     doc = (root / "INTEGRATION.md").read_text()
     assert int(re.search(r"_KSANA_SAGE_ABI = (\d+)", doc).group(1)) == abi == _capi.ABI_VERSION
+
+
+def test_argument_validation_under_the_host_address_sanitizer():
+    """``host_args_check`` drives the C ABI's validation paths from C++ with AddressSanitizer on the host pass of every
+    source: shapes, strides, the prep descriptor and its host-resident grid sizes are read under the sanitizer, and no
+    call reaches a device.  Built by ``__graft_entry__.build()``; rebuilt here when a source is newer (about a minute)."""
+    from ksanadit_amd import build_host_check as hc
+    from ksanadit_amd.build import CSRC
+
+    sources = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list(CSRC.glob("*.cpp")) + \
+        [Path(__file__).resolve().parent.parent / "include" / "ksana_sage_hip.h"]
+    if not hc.EXE_PATH.exists() or hc.EXE_PATH.stat().st_mtime < max(f.stat().st_mtime for f in sources):
+        hc.build_host_check(verbose=False)
+    r = hc.run_host_check()
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "0 failed" in r.stdout and "AddressSanitizer" not in r.stderr
