@@ -212,6 +212,24 @@ def other_workloads(sage_ops, dev, pwl, iters=7):
                        "quantizer_ms": round(ev[0].elapsed_time(ev[1]), 4)}
         del q, k, v, ws, out
         torch.cuda.empty_cache()
+    # Head size 64 (no BASELINE model has it; the backend interface serves it): the headline shape's token count
+    d64 = Workload("wan14b_480p_head_size_64", 1008, 1, 40, 32760)
+    q, k, v = device_inputs(d64, dev)
+    q, k, v = (t[..., :64].contiguous() for t in (q, k, v))
+    ws = sage_ops.workspace_for(q, k)
+    out = torch.empty_like(q)
+    sage_ops.quant_q(q, ws, 64**-0.5), sage_ops.quant_k(k, ws, True), sage_ops.quant_v(v, ws)
+    times = time_attention(sage_ops, ws, out, iters, pwl_exp2=pwl)
+    wide = pctl(time_attention(sage_ops, ws, out, iters, tile_skip=True), 0.5) if not pwl else None
+    ms = pctl(times, 0.5)
+    flops = 4.0 * d64.B * d64.H * d64.L * d64.L * 64
+    res[d64.name] = {"shape": f"B={d64.B} H={d64.H} L={d64.L} D=64", "attn_kernel_ms": spread(times),
+                     "attn_kernel_tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                     "frac_of_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                     "attn_kernel_ms_full_width_code": None if wide is None else round(wide, 4),
+                     "note": "operands zero-extended to 128 channels; the matrix instructions cover the lower 64 only (the upper 64 repeat them after the Hadamard transform)"}
+    del q, k, v, ws, out
+    torch.cuda.empty_cache()
     # Peaked attention, made on purpose: the headline distributions with q scaled by 4 (every score 4 times as far from
     # its row's mean), with and without the tile skip (KSANA_SAGE_FLAG_TILE_SKIP: same bits, see the header)
     if not pwl:

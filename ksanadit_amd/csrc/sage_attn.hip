@@ -58,8 +58,15 @@ struct WgShape {
   // one ring; with two rings everything issued in this step and the one before
   static constexpr int kInFlight = kTwoRings ? 2 * kCopies : kCopies * (kAhead - 2);
 };
-constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f
+constexpr int kMagicI = 0x4B400000;       // bits of 12582912.0f = 1.5 * 2^23: fp32 values are 1 apart there
 constexpr float kMagicF = 12582912.0f;
+// Head size 64 runs on rows whose upper 64 channels are zeros before the Hadamard transform - and a copy of the lower
+// 64 after it (H128 [x; 0] = [H64 x; H64 x]): the dot product over 128 channels is twice the one over the lower 64.
+// The kernel then multiplies the lower half only and starts its accumulators at 1.5 * 2^24, where fp32 values are 2
+// apart: the bits read as fp32 are 25165824 + 2 * dot, the full product, with no instruction spent on the doubling
+// (|dot| <= 127 * 127 * 64 < 2^21).
+constexpr int kMagicI2 = 0x4BC00000;      // bits of 25165824.0f = 1.5 * 2^24
+constexpr float kMagicF2 = 25165824.0f;
 // P is scaled by 2^6 before the e4m3 cast, and the reference point of a row (its "running maximum") is moved only when
 // a tile's maximum exceeds it by more than kLazyMax octaves: probabilities then reach 2^(6 + 2.7) = 416 < 448, the
 // largest e4m3 value, and the accumulators are rescaled in a few per cent of the steps instead of up to half of them
@@ -125,13 +132,15 @@ __device__ __forceinline__ void store4(uint16_t* dst, float a, float b, float c,
   *reinterpret_cast<uint2*>(dst) = half4<DT>(a, b, c, d);
 }
 
-// S^T tile (64 keys x 32 queries) of one wave: two 32-key sub-tiles, four 32-channel steps.
+// S^T tile (64 keys x 32 queries) of one wave: two 32-key sub-tiles, kG 32-channel steps (the channel groups that
+// hold data: 4, or 2 for head size 64, whose upper 64 channels are zeros on both sides).
+template <int kG>
 __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const v4i (&qf)[4], const v16i& magic,
                                         v16i (&acc)[2]) {
   acc[0] = magic;
   acc[1] = magic;
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
+  for (int s = 0; s < kG; ++s) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const v4i kf = *reinterpret_cast<const v4i*>(k_stage + ((t * 4 + s) * 64 + lane) * 16);
@@ -143,7 +152,10 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
 // kSplit: the workgroup takes one of `p.n_split` equal runs of key tiles of its (head, query block) and leaves
 // unnormalised accumulators, running maxima and row sums in the workspace for sage_attn_merge_kernel.  Used for
 // the workgroups beyond the last full round of the chip, which would otherwise hold it for a whole round alone.
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW, bool kTileSkip>
+// kG: 32-channel groups the matrix instructions cover - 4, or 2 when the head size is 64 (rows run zero-extended to
+// 128 channels and the operands keep their layout; see kMagicI2 for what is left out and why nothing is lost; the
+// result equals the full-width code's up to the rounding of one constant in the exponent).
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW, bool kTileSkip, int kG>
 __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg,
                                                                                    int n_wg, int wg_per_xcd) {
   static_assert(!(kSparse && kSplit), "the key split is built for the dense loop only");
@@ -152,6 +164,9 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   constexpr int kThreadsAttn = Shape::kThreads, kRowsWg = Shape::kRows, kStages = Shape::kStages, kAhead = Shape::kAhead;
   constexpr int kListMax = kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4;
   static_assert(!(kTileSkip && kPwlExp), "the piecewise-linear code formula has its own zero point: no tiles are skipped there");
+  static_assert(kG == 4 || kG == 2, "128 channels, or 64 zero-extended");
+  constexpr int kMagicBits = kG == 4 ? kMagicI : kMagicI2;
+  constexpr float kMagicVal = kG == 4 ? kMagicF : kMagicF2;
   int wg, split = 0;
   if constexpr (kSplit) {
     const int item = blockIdx.x / p.n_split;
@@ -225,7 +240,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   if (active) {
     const int8_t* qrow = p.q_i8 + ((int64_t)bh * p.lq_pad + q0 + l32) * kD + 16 * hh;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const v4i*>(qrow + 32 * s);
+    for (int s = 0; s < 4; ++s) qf[s] = s < kG ? *reinterpret_cast<const v4i*>(qrow + 32 * s) : v4i{0, 0, 0, 0};
     qs = p.q_scale[(int64_t)bh * p.lq_pad + q0 + l32];  // one scale per query row = per lane
   } else {
 #pragma unroll
@@ -259,7 +274,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   v16i magic;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    int m = kMagicI;
+    int m = kMagicBits;
     pin(m);
     magic[r] = m;
   }
@@ -393,7 +408,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     for (int r = 0; r < 16; ++r) {
       // all-ones where the key lies beyond the row
       const int beyond = (row_local - 4 * hh - (32 * t + 8 * (r >> 2) + (r & 3))) >> 31;
-      blk[r] = (blk[r] & ~beyond) | ((kMagicI - (1 << 22)) & beyond);
+      blk[r] = (blk[r] & ~beyond) | ((kMagicBits - (1 << 22)) & beyond);
     }
     return blk;
   };
@@ -563,9 +578,12 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     const v8i vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf, pf, oacc[dt], 0, 0, 0, 0, 0, 0);
   };
+  // S^T chunk i of a step is (channel step i / 2, key half i % 2); the chunks of channel steps without data carry only
+  // their share of the probabilities
+  auto has_qk = [](int i) { return i >= 0 && i < 8 && (i >> 1) < kG; };
 
   v16i s_a[2], s_b[2];
-  qk_tile(k_slot(0), lane, qf, magic, s_a);
+  qk_tile<kG>(k_slot(0), lane, qf, magic, s_a);
   // two rings: step 0 requests K tile kStages into the slot of K tile 0, which every wave must have read by then
   if constexpr (Shape::kTwoRings) __builtin_amdgcn_s_barrier();
   if (diag_at(0)) causal_scores(s_a);
@@ -599,7 +617,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     // dependent scalar work below, so their LDS latency is hidden behind it
     kf[0] = k_frag(0);
     kf[1] = k_frag(1);
-    kf[2] = k_frag(2);
+    kf[2] = k_frag(2);  // (kG >= 2: chunks 0 .. 3 always exist)
     const float ks_nxt = s_ks[min(j + 1, n_tiles - 1)];
     const bool mine = mine_at(j);
     issue_copy(j);
@@ -607,7 +625,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     // row sums of tile j-1: 64 matrix cycles that run under the max finalisation below
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_prev, lacc, 0, 0, 0, 0, 0, 0);
     const float sc = qs * ks_cur;
-    const float mneg = -kMagicF * sc;
+    const float mneg = -kMagicVal * sc;
     // a tile this wave's mask row does not ask for leaves the running maximum alone (wave-uniform
     // branch); its probabilities are zeroed where they are packed
     alpha_prev = mine ? update_max(mx_cur, sc, mneg) : 1.0f;
@@ -632,11 +650,12 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int s = i >> 1, t = i & 1;
-      if (i + 3 < 8)
-        kf[(i + 3) & 3] = k_frag(i + 3);
-      else
+      if (i + 3 < 8) {
+        if (has_qk(i + 3)) kf[(i + 3) & 3] = k_frag(i + 3);
+      } else if (i + 3 - 8 < kG) {
         vf[i + 3 - 8] = v_frag(i + 3 - 8);
-      s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i & 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
+      }
+      if (has_qk(i)) s_nxt[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i & 3], qf[s], s == 0 ? magic : s_nxt[t], 0, 0, 0);
       if constexpr (kPwlExp) {
         unsigned w = (i & 1) ? (unsigned)pf[i >> 1] : 0u;
         w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(__int_as_float(s_cur[0][2 * i]), scp, cp), (2 * i) & 3, w);
@@ -666,8 +685,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     // the max reduction of tile j+1, whose S^T MFMAs were issued at least one chunk ago]
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
-      if (dt == 0) vf[3] = v_frag(3);
-      oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
+      if (dt == 0 && kG == 4) vf[3] = v_frag(3);
+      if (dt < kG) oacc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[dt], pf_prev, oacc[dt], 0, 0, 0, 0, 0, 0);
       int w = 0;
       if (!nothing) w = pack4(s_cur[1][4 * dt], s_cur[1][4 * dt + 1], s_cur[1][4 * dt + 2], s_cur[1][4 * dt + 3], scp, cp);
       pin(w);
@@ -708,7 +727,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     const uint8_t* vst = v_slot(n_main - 1);
     const v8i pf_last = (n_main & 1) ? pf_y : pf_x;  // written by the last step
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf_last);
+    for (int dt = 0; dt < kG; ++dt) pv_slice(vst, dt, pf_last);
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf_last, lacc, 0, 0, 0, 0, 0, 0);
   }
   if (has_tail && mine_at(n_tiles - 1)) {  // ragged last tile, not pipelined: mask keys >= lk
@@ -719,10 +738,10 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int key = j * kBlkK + 32 * t + 8 * (r >> 2) + 4 * hh + (r & 3);
-        if (key >= lk) s_cur[t][r] = kMagicI - (1 << 22);  // below every real score
+        if (key >= lk) s_cur[t][r] = kMagicBits - (1 << 22);  // below every real score
       }
     const float sc = qs * s_ks[jj];
-    const float mneg = -kMagicF * sc;
+    const float mneg = -kMagicVal * sc;
     scale_o(update_max(lane_max(s_cur), sc, mneg));
     const float c = ((kPwlExp ? kPShiftPwl : kPShift) - m_run) + mneg;
     const float scp = kPwlExp ? 8.0f * sc : sc;
@@ -745,7 +764,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     if (diag_at(jj)) causal_probs(pf);
     const uint8_t* vst = v_slot(jj);
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) pv_slice(vst, dt, pf);
+    for (int dt = 0; dt < kG; ++dt) pv_slice(vst, dt, pf);
     lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, lacc, 0, 0, 0, 0, 0, 0);
   }
 
@@ -754,7 +773,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     const int row = wave * 32 + l32;
     float* po = p.split_o + ((int64_t)blockIdx.x * kAttnQPerWg + row) * kD;
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < kG; ++dt)
 #pragma unroll
       for (int g = 0; g < 4; ++g)
         *reinterpret_cast<float4*>(po + 32 * dt + 8 * g + 4 * hh) =
@@ -781,14 +800,14 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   const float4* vm4 = reinterpret_cast<const float4*>(s_vs + kD);
   float4 s4a[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) s4a[i] = vs4[(32 * (i >> 2) + 8 * (i & 3) + 4 * hh) >> 2];
+  for (int i = 0; i < 4 * kG; ++i) s4a[i] = vs4[(32 * (i >> 2) + 8 * (i & 3) + 4 * hh) >> 2];
   const float2 mm = reinterpret_cast<const float2*>(s_vs + kD)[lane];
   const bool has_mean = __any(mm.x != 0.0f || mm.y != 0.0f);  // wave-uniform
   __syncthreads();  // waves that ended early (no query rows) do not count
   uint8_t* stage = smem + wave * (32 * kPitch);
   if (!has_mean) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < 4 * kG; ++i) {
       const int dt = i >> 2, g = i & 3;
       const int d = 32 * dt + 8 * g + 4 * hh;
       const float4 s4 = s4a[i];
@@ -798,7 +817,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < 4 * kG; ++i) {
       const int dt = i >> 2, g = i & 3;
       const int d = 32 * dt + 8 * g + 4 * hh;
       const float4 s4 = s4a[i];
@@ -814,7 +833,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   for (int i = 0; i < 8; ++i) {
     const int idx = i * 64 + lane, r = idx >> 4, c = idx & 15;  // row r of the wave, 16-byte piece c of it
     const uint4 piece = *reinterpret_cast<const uint4*>(stage + r * kPitch + 16 * c);
-    if (q0 + r < p.Lq && 8 * c < p.d_out) *reinterpret_cast<uint4*>(obase + (int64_t)(q0 + r) * p.o.sL + 8 * c) = piece;
+    if (q0 + r < p.Lq && 8 * c < p.d_out && 8 * c < 32 * kG) *reinterpret_cast<uint4*>(obase + (int64_t)(q0 + r) * p.o.sL + 8 * c) = piece;
   }
 }
 
@@ -864,7 +883,7 @@ constexpr size_t max_lds() {
                  : WgShape<kW>::kRingBytes + 1024 + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
 }
 
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8, bool kTileSkip = false>
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8, bool kTileSkip = false, int kG = 4>
 hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
   // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
@@ -875,12 +894,12 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg,
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   if (!requested[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip>),
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip, kG>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_lds<kSparse, kW>());
     if (e != hipSuccess) return e;
     requested[dev].store(true, std::memory_order_release);
   }
-  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip, kG><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
 }
 
@@ -888,6 +907,11 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg,
 template <bool kSparse, bool kSplit, int kW>
 hipError_t launch_shape(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd, hipStream_t s) {
   const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
+  // head size 64: the matrix instructions on the zero halves are left out (plain exact-exponential calls; the other
+  // variants run the full-width code on the same operands, which gives the same bits)
+  if (p.exact_exp2 && !p.tile_skip && p.d_out <= 64)
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, false, 2>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, false, 2>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   if (p.exact_exp2 && p.tile_skip)
     return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
                 : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);

@@ -49,7 +49,7 @@ def p_to_e4m3(x: torch.Tensor, exact_exp2: bool = True) -> torch.Tensor:
 
 
 def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype, causal=False, online=True,
-                         exact_exp2=True, k_lens=None, block_mask=None, v_mean=None, key_split=None):
+                         exact_exp2=True, k_lens=None, block_mask=None, v_mean=None, key_split=None, magic=12582912.0):
     """Logical-layout operands ([B,H,L,D] etc.) -> O [B, Lq, H, D] in ``out_dtype``.
 
     ``online=True`` walks the keys in tiles of ``BLKK`` like the kernel: the running row max
@@ -64,6 +64,10 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
     the 256-row query blocks numbered ``first_workgroup`` and up (numbering: ``(b * H + h) * ceil(Lq/256) + block``)
     into ``runs`` equal runs of key tiles, walks each run on its own and merges the partial results; probabilities are
     then rounded relative to the run's own running maximum, which this mirrors.
+    ``magic``: the constant the kernel's integer accumulators start from, read as fp32: 1.5 * 2**23 - or 1.5 * 2**24 where
+    the kernel multiplies only the lower 64 channels of rows that were zero-extended from head size 64 (after the
+    Hadamard transform the upper 64 repeat the lower 64, and at 2**24 the fp32 grid doubles the half product for free).
+    The value changes the rounding of the exponent's constant term, nothing else.
     ``causal``: row ``i`` sees keys ``[0, i]`` (for ``Lq != Lk`` too: the triangle sits in the top left corner, as
     torch's ``is_causal`` puts it); in the online form a row sits out the tiles that start after it and sees a prefix
     of the tile that holds its own position.
@@ -104,8 +108,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                 #   m   = max(m, fma(x_f_max, sc, -MAGIC * sc))
                 #   c   = (SHIFT - m) + (-MAGIC * sc)   fp32, in this order
                 #   exponent = fma(x_f, sc, c)          (pwl: fma(x_f, 8 sc, fma(8, c, 55.5)))
-                magic = 12582912.0
-                x_f = (s_int + magic).to(torch.float32)  # exact: |dot| < 2**22
+                x_f = (s_int + magic).to(torch.float32)  # exact: |dot| < 2**22 (and even where magic is 1.5 * 2**24)
                 rows = torch.arange(Lq)[:, None]
 
                 def walk(key_from, key_to):
@@ -134,7 +137,7 @@ def sage_emul_from_quant(q_i8, q_scale, k_i8, k_scale, v_fp8, v_scale, out_dtype
                     xt = x_f[:, j0:j1]
                     mneg = -(magic * sc)  # fp32
                     # a key the row may not see scores magic - 2**22, below every real dot product
-                    xt_max = xt if allow is None else torch.where(allow, xt, torch.tensor(magic - 4194304.0))
+                    xt_max = xt if allow is None else torch.where(allow, xt, torch.tensor(magic - (4194304.0 if magic < 2.0**24 else 8388608.0)))
                     m_tile = (xt_max.amax(dim=1, keepdim=True).double() * sc.double() + mneg.double()).float()  # fma
                     lazy = torch.tensor(LAZY_MAX if exact_exp2 else LAZY_MAX_PWL, dtype=torch.float32)
                     m_new = torch.where(m_tile > m + lazy, m_tile, m)
