@@ -616,6 +616,7 @@ def sageattn(
     out_dtype: torch.dtype | None = None,
     smooth_v: bool = False,
     q_lens=None,
+    tile_skip: bool = False,
 ) -> torch.Tensor:
     """Quantized attention, ``[B, L, H, D]`` ("NHD") or ``[B, H, L, D]`` ("HND") in and out.
 
@@ -633,7 +634,10 @@ def sageattn(
     (ksana/models/wan/wan_model.py:197-204), done in the kernel's epilogue from the fp32 accumulators.
 
     ``pwl_exp2=True`` computes the e4m3 code of every probability directly (exp2 with a
-    piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate."""
+    piecewise-linear mantissa, no transcendental): about 1.2x faster, slightly less accurate.
+    ``tile_skip=True`` (exact exponential only): see ``attn_fwd``; same bits, faster on sharply peaked attention."""
+    if tile_skip and pwl_exp2:
+        raise ValueError("tile_skip goes with the exact exponential only")
     if tensor_layout not in ("NHD", "HND"):
         raise ValueError(f"tensor_layout {tensor_layout!r} unknown")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -657,6 +661,7 @@ def sageattn(
     _log_demotion_once()
     kl = _k_lens_arg(k_lens, B, q.device)
     flags = (_capi.FLAG_PWL_EXP2 if pwl_exp2 else 0) | (_capi.FLAG_SMOOTH_V if smooth_v else 0)
+    flags |= _capi.FLAG_TILE_SKIP if tile_skip else 0
     if prep is not None:
         _check_qwen_rows(prep, Lq)
         _check_qwen_rows(prep, k.shape[1])
