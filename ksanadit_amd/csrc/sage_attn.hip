@@ -155,10 +155,15 @@ __device__ __forceinline__ void qk_tile(const uint8_t* k_stage, int lane, const 
 // kG: 32-channel groups the matrix instructions cover - 4, or 2 when the head size is 64 (rows run zero-extended to
 // 128 channels and the operands keep their layout; see kMagicI2 for what is left out and why nothing is lost; the
 // result equals the full-width code's up to the rounding of one constant in the exponent).
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW, bool kTileSkip, int kG>
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW, bool kTileSkip, int kG, bool kCausal>
 __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel(const AttnParams p, int n_qwg,
                                                                                    int n_wg, int wg_per_xcd) {
   static_assert(!(kSparse && kSplit), "the key split is built for the dense loop only");
+  static_assert(kSparse || !kCausal, "causal calls run through the tile list");
+  // kCausal == false: the caller vouches that p.causal is 0, and everything that serves the diagonal (the per-wave
+  // last tile, 32 lane masks held in scalar registers, the selects that blank a wave's probabilities past its rows)
+  // is compiled out of the key loop
+  const bool causal = kCausal && p.causal;
   static_assert(!kSplit || kW == 8, "the key split is built for 256-row workgroups");
   using Shape = WgShape<kW>;
   constexpr int kThreadsAttn = Shape::kThreads, kRowsWg = Shape::kRows, kStages = Shape::kStages, kAhead = Shape::kAhead;
@@ -183,7 +188,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   const int bh = wg / n_qwg;
   int qwg = wg - bh * n_qwg;
   // causal: the later a query block, the more key tiles it walks - start the long ones first
-  if (kSparse && p.causal) qwg = n_qwg - 1 - qwg;
+  if (kSparse && causal) qwg = n_qwg - 1 - qwg;
   const int b = bh / p.Hq, h = bh - b * p.Hq;
   const int bhk = b * p.Hkv + h / (p.Hq / p.Hkv);
 
@@ -301,7 +306,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   int* s_list = reinterpret_cast<int*>(s_ks + kListMax);
   int n_tiles = nkb;  // loop length: list entries with a mask, key tiles without
   // a wave's 32 rows start at a multiple of 32, so exactly one 64-key tile holds their diagonal
-  const int my_last = (kSparse && p.causal) ? (q0 >> 6) : 0x7fffffff;
+  const int my_last = (kSparse && causal) ? (q0 >> 6) : 0x7fffffff;
   if constexpr (kSparse) {
     if (wave == 0) {
       const int nqm = (p.Lq + kMaskBlkQ - 1) / kMaskBlkQ;
@@ -309,7 +314,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
       constexpr int kMaskRows = kRowsWg / kMaskBlkQ;  // mask rows a workgroup covers: 2 or 1
       const int8_t* m0 = masked ? p.block_mask + b * p.mask_sB + h * p.mask_sH + (int64_t)(kMaskRows * qwg) * p.nkb : nullptr;
       const bool two = kMaskRows == 2 && 2 * qwg + 1 < nqm;
-      const int wg_tiles = p.causal ? min(nkb, ((qwg * kRowsWg + kRowsWg - 1) >> 6) + 1) : nkb;
+      const int wg_tiles = causal ? min(nkb, ((qwg * kRowsWg + kRowsWg - 1) >> 6) + 1) : nkb;
       int base = 0;
       // eight chunks of 64 tiles at a time: their mask bytes are requested together, so a list of 512 tiles costs
       // one memory latency instead of eight
@@ -368,7 +373,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // loop then compares loop positions instead of looking list entries up.
   int n_mine = n_tiles, jdiag = -1;  // wave-uniform
   if constexpr (kSparse) {
-    if (p.causal) {
+    if (causal) {
       if (p.block_mask == nullptr) {  // the list is 0, 1, 2, ...
         n_mine = min(n_tiles, my_last + 1);
       } else {
@@ -390,7 +395,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   };
   auto mine_at = [&](int jj) -> bool {
     if constexpr (kSparse) {
-      if constexpr (kW == 4) return jj < n_mine;  // one mask row per workgroup: every listed tile is wanted
+      if constexpr (kW == 4 && !kCausal) return true;  // one mask row per workgroup: every listed tile is wanted
+      if constexpr (kW == 4) return jj < n_mine;
       const int e = __builtin_amdgcn_readfirstlane(s_list[jj]);
       return ((e >> (16 + (wave >> 2))) & 1) != 0 && jj < n_mine;
     }
@@ -398,7 +404,7 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   };
   // causal only: list position jj holds the tile on this wave's diagonal
   auto diag_at = [&](int jj) -> bool {
-    if constexpr (kSparse) return jj == jdiag;
+    if constexpr (kSparse && kCausal) return jj == jdiag;
     return false;
   };
   // scores of keys beyond the row's own position drop below every real score ...
@@ -447,18 +453,35 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   };
   // clamped: past the end the last tile is copied again into a slot nobody reads any more,
   // which keeps the loop free of branches and the outstanding-copy count constant
-  auto copy_half = [&](const uint8_t* src, int tile, uint8_t* dst) {
-    const int jl = tile_of(min(tile, n_tiles - 1));
+  auto copy_tile_half = [&](const uint8_t* src, int jl, uint8_t* dst) {  // jl: key tile number, wave-uniform
 #pragma unroll
     for (int c = 0; c < 8 / kW; ++c) {  // this wave's 1 KiB slices of the tile: slice c * kW + wave
       const int slice = c * kW + wave;
       lds_copy16(src + (int64_t)jl * kTileBytes, (unsigned)(slice * 64 + lane) * 16, dst + slice * 1024);
     }
   };
+  auto copy_half = [&](const uint8_t* src, int tile, uint8_t* dst) {
+    copy_tile_half(src, tile_of(min(tile, n_tiles - 1)), dst);
+  };
+  // With a tile list, the key tiles behind the loop positions whose copies the next steps issue are kept in scalar
+  // registers: looked up in the step, a list entry costs an LDS read whose wait also drains the operand reads
+  // requested just before it.  ahead[i] = tile at position j + kAhead + i for the step j about to run; a step
+  // fetches the one entry that enters the window (position j + 1 + kAheadK) and takes it over at its end.
+  constexpr int kWindow = Shape::kAheadK - kAhead + 1;
+  int ahead[kWindow];
+  if constexpr (kSparse) {
+#pragma unroll
+    for (int i = 0; i < kWindow; ++i) ahead[i] = tile_of(min(kAhead + i, n_tiles - 1));
+  }
   // the copies of loop step j (step -1: nothing; the prologue below brings the first tiles in)
   auto issue_copy = [&](int j) {
-    copy_half(v_src, j + kAhead, v_slot(j + kAhead));  // first: it is awaited first
-    copy_half(k_src, j + Shape::kAheadK, k_slot(j + Shape::kAheadK));
+    if constexpr (kSparse) {
+      copy_tile_half(v_src, ahead[0], v_slot(j + kAhead));
+      copy_tile_half(k_src, ahead[kWindow - 1], k_slot(j + Shape::kAheadK));
+    } else {
+      copy_half(v_src, j + kAhead, v_slot(j + kAhead));  // first: it is awaited first
+      copy_half(k_src, j + Shape::kAheadK, k_slot(j + Shape::kAheadK));
+    }
   };
   // wait until every copy except the newest Shape::kInFlight has landed, then meet the other waves.
   // Plain s_barrier: a fence here would drain ALL copies and undo the prefetch.
@@ -502,7 +525,9 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     // same copy / barrier sequence as the active waves
     if constexpr (Shape::kTwoRings) __builtin_amdgcn_s_barrier();
     for (int j = 0; j < n_main; ++j) {
-      issue_copy(j);
+      // (looks the tiles up where they are needed: a wave without rows has nothing an LDS wait could hold up)
+      copy_half(v_src, j + kAhead, v_slot(j + kAhead));
+      copy_half(k_src, j + Shape::kAheadK, k_slot(j + Shape::kAheadK));
       tile_barrier();
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -619,6 +644,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     kf[1] = k_frag(1);
     kf[2] = k_frag(2);  // (kG >= 2: chunks 0 .. 3 always exist)
     const float ks_nxt = s_ks[min(j + 1, n_tiles - 1)];
+    int entering = 0;  // the list entry the next step's window gains; it arrives with the operands above
+    if constexpr (kSparse) entering = s_list[min(j + 1 + Shape::kAheadK, n_tiles - 1)];
     const bool mine = mine_at(j);
     issue_copy(j);
     if (__any(alpha_prev < 1.0f)) scale_o(alpha_prev);
@@ -698,6 +725,9 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
     mx_cur = max(max(pm[0], pm[1]), max(pm[2], pm[3]));
     ks_cur = ks_nxt;
     if constexpr (kSparse) {
+#pragma unroll
+      for (int i = 0; i + 1 < kWindow; ++i) ahead[i] = ahead[i + 1];
+      ahead[kWindow - 1] = __builtin_amdgcn_readfirstlane(entering) & 0xffff;
       if (!mine) {  // wave-uniform and rare: a tile this wave's row does not take part in contributes nothing
 #pragma unroll
         for (int i = 0; i < 8; ++i) pf[i] = 0;
@@ -883,7 +913,7 @@ constexpr size_t max_lds() {
                  : WgShape<kW>::kRingBytes + 1024 + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
 }
 
-template <int DT, bool kPwlExp, bool kSparse, bool kSplit = false, int kW = 8, bool kTileSkip = false, int kG = 4>
+template <int DT, bool kPwlExp, bool kSparse, bool kSplit, int kW, bool kCausal, bool kTileSkip = false, int kG = 4>
 hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd,
                           hipStream_t s) {
   // more than 64 KiB of dynamic LDS has to be requested per kernel, once per device
@@ -894,32 +924,32 @@ hipError_t launch_variant(const AttnParams& p, dim3 grid, size_t lds, int n_qwg,
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
   if (!requested[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip, kG>),
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip, kG, kCausal>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_lds<kSparse, kW>());
     if (e != hipSuccess) return e;
     requested[dev].store(true, std::memory_order_release);
   }
-  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip, kG><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
+  sage_attn_fwd_kernel<DT, kPwlExp, kSparse, kSplit, kW, kTileSkip, kG, kCausal><<<grid, dim3(kW * 64), lds, s>>>(p, n_qwg, n_wg, wg_per_xcd);
   return hipGetLastError();
 }
 
 // the (dtype, exp2 form, tile skip) instantiations behind one (mask, split, workgroup shape) choice
-template <bool kSparse, bool kSplit, int kW>
+template <bool kSparse, bool kSplit, int kW, bool kCausal = false>
 hipError_t launch_shape(const AttnParams& p, dim3 grid, size_t lds, int n_qwg, int n_wg, int wg_per_xcd, hipStream_t s) {
   const bool bf16 = p.o.dtype == KSANA_SAGE_BF16;
   // head size 64: the matrix instructions on the zero halves are left out (plain exact-exponential calls; the other
   // variants run the full-width code on the same operands, which gives the same bits)
   if (p.exact_exp2 && !p.tile_skip && p.d_out <= 64)
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, false, 2>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, false, 2>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, kCausal, false, 2>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, kCausal, false, 2>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   if (p.exact_exp2 && p.tile_skip)
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, kCausal, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, kCausal, true>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   if (p.exact_exp2)
-    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
-                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
-  return bf16 ? launch_variant<KSANA_SAGE_BF16, true, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
-              : launch_variant<KSANA_SAGE_FP16, true, kSparse, kSplit, kW>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
+    return bf16 ? launch_variant<KSANA_SAGE_BF16, false, kSparse, kSplit, kW, kCausal>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+                : launch_variant<KSANA_SAGE_FP16, false, kSparse, kSplit, kW, kCausal>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
+  return bf16 ? launch_variant<KSANA_SAGE_BF16, true, kSparse, kSplit, kW, kCausal>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s)
+              : launch_variant<KSANA_SAGE_FP16, true, kSparse, kSplit, kW, kCausal>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
 }
 
 // compute units of the current device (the size of one round of workgroups: one workgroup per unit)
@@ -977,7 +1007,9 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
     const int n_wg = p.B * p.Hq * n_qwg;
     const int wg_per_xcd = (n_wg + 7) / 8;
     const dim3 grid(wg_per_xcd * 8);
-    if (sparse) return launch_shape<true, false, 4>(p, grid, max_lds<true, 4>(), n_qwg, n_wg, wg_per_xcd, s);
+    if (sparse)
+      return p.causal ? launch_shape<true, false, 4, true>(p, grid, max_lds<true, 4>(), n_qwg, n_wg, wg_per_xcd, s)
+                      : launch_shape<true, false, 4, false>(p, grid, max_lds<true, 4>(), n_qwg, n_wg, wg_per_xcd, s);
     const size_t lds = WgShape<4>::kRingBytes + 1024 + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
     return launch_shape<false, false, 4>(p, grid, lds, n_qwg, n_wg, wg_per_xcd, s);
   }
@@ -985,7 +1017,8 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const int n_wg = p.B * p.Hq * n_qwg;
   const int wg_per_xcd = (n_wg + 7) / 8;
   const dim3 grid(wg_per_xcd * 8);
-  if (sparse) return launch_shape<true, false, 8>(p, grid, max_lds<true, 8>(), n_qwg, n_wg, wg_per_xcd, s);
+  // (beyond 65 536 keys with a mask: one instantiation serves causal and plain calls)
+  if (sparse) return launch_shape<true, false, 8, true>(p, grid, max_lds<true, 8>(), n_qwg, n_wg, wg_per_xcd, s);
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
   const size_t lds = WgShape<8>::kRingBytes + 1024 + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));
   // The workgroups beyond the last full round of the chip (one workgroup per compute unit) would hold it for a
