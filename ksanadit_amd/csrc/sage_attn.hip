@@ -409,7 +409,10 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   };
   // scores of keys beyond the row's own position drop below every real score ...
   auto causal_half = [&](v16i blk, int t) -> v16i {
-    const int row_local = (q0 & 63) + l32;
+    // (pinned: the comparisons below are the same in every step, and hoisted out of the key loop they would sit in
+    // 32 scalar register pairs for a block that runs once per wave)
+    int row_local = (q0 & 63) + l32;
+    pin(row_local);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       // all-ones where the key lies beyond the row
@@ -425,7 +428,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // ... and their probability bytes are cleared outright (code 0 is +0.0 in e4m3), so that a row
   // whose scale is zero does not count them either
   auto causal_probs = [&](v8i& pf) {
-    const int row_local = (q0 & 63) + l32;
+    int row_local = (q0 & 63) + l32;
+    pin(row_local);
 #pragma unroll
     for (int w = 0; w < 8; ++w) {
       // bytes of the first min(max(n, 0), 4) keys of this dword stay
