@@ -353,21 +353,21 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
       write_zero_rows();
       return;
     }
-    for (int i = tid; i < n_tiles; i += kThreadsAttn) s_ks[i] = ks_ptr[s_list[i] & 0xffff];
   }
-  // the head's K scales (dense: in tile order) and V scales / means go to LDS; without a tile list this waits until
-  // the first tile copies are on their way, so that the loads' latencies overlap
+  // the head's K scales (in loop order: tile order, or the list's) and V scales / means go to LDS, once the first
+  // tile copies are on their way, so that the loads' latencies overlap
   auto fill_scales = [&]() {
     // the V value is requested first and stored last: written where it is loaded, its load would only go out after
     // the K scales' loads had been awaited - a second memory latency in every workgroup's set-up
     float vsm = 0.0f;
     if (tid < 2 * kD) vsm = tid < kD ? p.v_scale[(int64_t)bhk * kD + tid] : p.v_mean[(int64_t)bhk * kD + tid - kD];
-    if constexpr (!kSparse) {
+    if constexpr (kSparse) {
+      for (int i = tid; i < n_tiles; i += kThreadsAttn) s_ks[i] = ks_ptr[s_list[i] & 0xffff];
+    } else {
       for (int i = tid; i < nkb; i += kThreadsAttn) s_ks[i] = ks_ptr[i];
     }
     if (tid < 2 * kD) s_vs[tid] = vsm;
   };
-  if constexpr (kSparse) fill_scales();
   // Causal calls: the list is in key order, so the entries this wave takes part in (tile <= the one on its diagonal)
   // are the first n_mine, and the diagonal tile, if listed, is the last of them.  Both are found once here; the key
   // loop then compares loop positions instead of looking list entries up.
@@ -496,9 +496,8 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // The compiler does not see the asynchronous copies in the memory-operation counter it models.  Every ordinary global
   // load of the set-up (Q fragments, scales) must therefore be known to have returned before the key loop starts:
   // left to itself the compiler would wait for "all but its n newest loads" at the first use of a loaded value
-  // inside the loop, and drain the copies issued since.  With a tile list the loads are awaited before the first copy;
-  // without one the first copies go out first (the tile numbers are known) and everything is awaited together.
-  if constexpr (kSparse) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  // inside the loop, and drain the copies issued since.  The first copies go out first and everything is awaited
+  // together.
   // The V^T slot of "tile -1" is read (times P = 0) by the first loop iteration: make it finite.
 #pragma unroll
   for (int c = 0; c < 8 / kW; ++c)
@@ -515,15 +514,9 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
       copy_half(v_src, t, v_slot(t));
     }
   }
-  if constexpr (!kSparse) {
-    fill_scales();
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the set-up's loads and, older than some of them, the copies
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  } else if constexpr (Shape::kTwoRings) {
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(Shape::kInFlight) : "memory");  // tiles 0, 1 visible
-  }
+  fill_scales();
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the set-up's loads and, older than some of them, the copies
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   if (!active) {
     // same copy / barrier sequence as the active waves
