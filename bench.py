@@ -403,7 +403,7 @@ def prep_quantizer_leg(sage_ops, w, q, k, v, ws, sm_scale, grid, dev, iters):
 
 def sla_leg(sage_ops, w, q, k, v, ws, dev, iters, topk=0.1):
     """Outside the timed step: the sparse-linear backend at the headline shape, part by part (HIP events): the block
-    map (block averages on HIP, then the reference's GEMM + topk + scatter), the block-sparse attention on that map,
+    map (block averages taken along by the quantizers of q and k, then scores + top-k), the block-sparse attention on that map,
     the linear branch with the block's linear layer and the final sum folded in (HIP), and - for scale - the same
     branch as the reference issues it (five torch kernels plus the layer plus the sum)."""
     from ksanadit_amd.backends import sage_sla
@@ -422,12 +422,16 @@ def sla_leg(sage_ops, w, q, k, v, ws, dev, iters, topk=0.1):
         return pctl([e[0].elapsed_time(e[1]) for e in ev], 0.5)
 
     proj = torch.nn.Linear(w.D, w.D, bias=True).to(dev).to(q.dtype)
-    sage_ops.quant_q(q, ws, w.D**-0.5)  # the legs before this one left other operands in the workspace
-    sage_ops.quant_k(k, ws, True)
+    sm = w.D**-0.5
+    # (the legs before this one left other operands in the workspace)
+    pq, pk = sage_ops.quant_qk_pooled(q, k, ws, sm)
     sage_ops.quant_v(v, ws)
-    bm, kept = sage_sla.topk_block_map(q, k, ws.k_mean, topk)
+    bm, kept = sage_sla.block_map_from_pooled(pq, pk, topk)
     out = torch.empty_like(q)
-    map_ms = timed(lambda: sage_sla.topk_block_map(q, k, ws.k_mean, topk))
+    # the block averages ride in the quantizers of q and k: what they add to those two, and the map kernel itself
+    plain_ms = timed(lambda: (sage_ops.quant_q(q, ws, sm), sage_ops.quant_k(k, ws, True)))
+    pooled_ms = timed(lambda: sage_ops.quant_qk_pooled(q, k, ws, sm))
+    map_ms = timed(lambda: sage_sla.block_map_from_pooled(pq, pk, topk))
     pool_ms = timed(lambda: (sage_ops.block_means(q, 128), sage_ops.block_means(k, 64, centre=ws.k_mean)))
     attn_ms = timed(lambda: sage_ops.attn_fwd(ws, out, block_mask=bm))
     with torch.no_grad():
@@ -447,8 +451,10 @@ def sla_leg(sage_ops, w, q, k, v, ws, dev, iters, topk=0.1):
     return {
         "what": "SageSLA backend, topk share %.2f: block map + block-sparse attention + linear branch (layer and sum folded in)" % topk,
         "kept_key_blocks": f"{kept} of {bm.shape[-1]}",
-        "block_map_ms": round(map_ms, 4),
-        "block_map_pooling_part_ms": round(pool_ms, 4),
+        "block_map_ms": round(map_ms + pooled_ms - plain_ms, 4),
+        "block_map_note": "scores + top-k kernel, plus what the block averages add to the quantizers of q and k they ride in",
+        "block_averages_in_quantizers_ms": round(pooled_ms - plain_ms, 4),
+        "block_averages_as_own_passes_ms": round(pool_ms, 4),
         "sparse_attn_ms": round(attn_ms, 4),
         "sparse_attn_tflops_on_kept_blocks": round(w.flops * kept / bm.shape[-1] / (attn_ms * 1e-3) / 1e12, 1),
         "linear_branch_ms": round(lin_ms, 4),

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define KSANA_SAGE_ABI_VERSION 19
+#define KSANA_SAGE_ABI_VERSION 20
 
 /* element types of q/k/v/o */
 #define KSANA_SAGE_BF16 0
@@ -253,6 +253,16 @@ int ksana_sage_quant_v_smooth(const void* v, int dtype, const int64_t v_strides[
  * Replaces the Triton kernel compress_kernel / mean_pool (sage_sla.py:43-75). */
 int ksana_sage_block_means(const void* x, int dtype, const int64_t strides[4], int B, int H, int L, int rows_per_block,
                            const float* centre, void* out, void* stream);
+
+/* ksana_sage_quant_q + ksana_sage_quant_k (smooth_k = 1) that take the sparse-linear backend's block averages along:
+ * pooled_q [B, Hq, ceil(Lq / 128), 128] and pooled_k [B, Hkv, ceil(Lk / 64), 128] (device, `dtype`, contiguous) come
+ * out bit for bit as ksana_sage_block_means(q, 128 rows) and ksana_sage_block_means(k, 64 rows, centre = the
+ * workspace's k_mean) give them - the quantizers' workgroups are those blocks - without reading q and k once more.
+ * Head size 128 only (KSANA_SAGE_ENOTSUP otherwise).  Replaces get_vanilla_qk_quant (sage_sla.py:202-204) together
+ * with compress_kernel / mean_pool on q and on k - mean(k) (sage_sla.py:43-81). */
+int ksana_sage_quant_qk_pooled(const void* q, const void* k, int dtype, const int64_t q_strides[4],
+                               const int64_t k_strides[4], const ksana_sage_shape* shape, float sm_scale,
+                               void* pooled_q, void* pooled_k, void* workspace, void* stream);
 
 /* The second half of get_block_map (sage_sla.py:83-90) in one kernel: score = pooled_q pooled_k^T as a tensor of the
  * blocks' dtype, then per query block ones at the `keep` key blocks with the largest scores (of equal scores the

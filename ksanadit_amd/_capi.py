@@ -11,7 +11,7 @@ import threading
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libksana_sage_hip.so"
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 BF16, FP16 = 0, 1
 OK, EINVAL, ENOTSUP, EHIP = 0, -1, -2, -3
@@ -39,6 +39,7 @@ EXPORTS = (
     "ksana_sage_attn_key_split",
     "ksana_sage_quant_status",
     "ksana_sage_block_means",
+    "ksana_sage_quant_qk_pooled",
     "ksana_sage_sla_workspace_bytes",
     "ksana_sage_sla_linear",
     "ksana_sage_sla_block_map",
@@ -119,6 +120,8 @@ def _declare(lib):
     lib.ksana_sage_quant_status.argtypes, lib.ksana_sage_quant_status.restype = [vp, sp, vp, ip, ip], i
     lib.ksana_sage_block_means.argtypes = [vp, i, st, i, i, i, i, vp, vp, vp]
     lib.ksana_sage_block_means.restype = i
+    lib.ksana_sage_quant_qk_pooled.argtypes = [vp, vp, i, st, st, sp, f, vp, vp, vp, vp]
+    lib.ksana_sage_quant_qk_pooled.restype = i
     lib.ksana_sage_sla_workspace_bytes.argtypes = [i, i, i, C.POINTER(C.c_uint64)]
     lib.ksana_sage_sla_workspace_bytes.restype = i
     lib.ksana_sage_sla_linear.argtypes = [vp, vp, vp, i, st, st, st, i, i, i, vp, vp, vp, st, vp, st, vp, vp]

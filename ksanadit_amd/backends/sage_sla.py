@@ -3,10 +3,10 @@
 Drop-in for ksana/operations/attention/backends/sage_sla.py:100-292.  Per call (unless ``dense_only``):
 
 1. a block map: q and the mean-centred k are averaged over blocks of 128 query rows / 64 keys (the reference's one
-   in-repo GPU kernel, ``compress_kernel`` / ``mean_pool``, sage_sla.py:43-75 - here the HIP kernel behind
-   ``ksana_sage_block_means``, which reads the ``[B, L, H, D]`` tensors as they are and takes k's mean from the
-   quantizer's workspace), the block averages are multiplied, and every query block keeps its ``topk`` share of the key
-   blocks with the largest products (sage_sla.py:78-90, 189);
+   in-repo GPU kernel, ``compress_kernel`` / ``mean_pool``, sage_sla.py:43-75 - here the averages ride in the
+   quantizers of q and k, whose workgroups are exactly those blocks: ``ksana_sage_quant_qk_pooled``; the stand-alone
+   kernel is ``ksana_sage_block_means``), the block averages are multiplied, and every query block keeps its ``topk``
+   share of the key blocks with the largest products (sage_sla.py:78-90, 189);
 2. block-sparse quantized attention over the kept blocks (sage_sla.py:196-271) - this package's masked kernel, which
    takes the int8 map as it is, on the operands quantized once for both steps;
 3. a linear-attention branch on softmax feature maps of q and k, passed through the block's ``proj_l`` layer, added
@@ -104,10 +104,9 @@ class SageSLAAttentionImpl(KsanaAttentionBackendImpl):
             query, key, value = (t.to(torch.bfloat16) for t in (query, key, value))
         # quantize once; the block map is built next to the quantized operands and drives the attention over them
         ws = sage_ops.workspace_for(query, key)
-        sage_ops.quant_q(query, ws, query.shape[-1] ** -0.5)
-        sage_ops.quant_k(key, ws, True)
+        pooled_q, pooled_k = sage_ops.quant_qk_pooled(query, key, ws, query.shape[-1] ** -0.5)  # averages ride along
         sage_ops.quant_v(value, ws)
-        block_map, kept = topk_block_map(query, key, ws.k_mean, self.topk)
+        block_map, kept = block_map_from_pooled(pooled_q, pooled_k, self.topk)
         o_sparse = sage_ops.attn_fwd(ws, torch.empty_like(query), block_mask=block_map)
         if isinstance(proj_l, torch.nn.Linear) and tuple(proj_l.weight.shape) == (query.shape[-1],) * 2:
             # the layer and the sum of the two branches ride along in the linear branch's second pass

@@ -99,6 +99,10 @@ int main() {
          KSANA_SAGE_EINVAL);
   EXPECT(ksana_sage_sla_block_map(fake, fake, KSANA_SAGE_BF16, 1, 2, 8, 2000, 3, reinterpret_cast<int8_t*>(fake), nullptr), KSANA_SAGE_ENOTSUP);
   EXPECT(ksana_sage_block_means(fake, KSANA_SAGE_BF16, st, 1, 2, 64, 48, nullptr, fake, nullptr), KSANA_SAGE_ENOTSUP);
+  ksana_sage_shape d64{1, 2, 2, 64, 64, 64};
+  EXPECT(ksana_sage_quant_qk_pooled(fake, fake, KSANA_SAGE_BF16, st, st, &d64, 0.1f, fake, fake, fake, nullptr), KSANA_SAGE_ENOTSUP);
+  EXPECT(ksana_sage_quant_qk_pooled(fake, fake, KSANA_SAGE_BF16, st, st, &s, 0.1f, fake, nullptr, fake, nullptr), KSANA_SAGE_EINVAL);
+  EXPECT(ksana_sage_quant_qk_pooled(fake, nullptr, KSANA_SAGE_BF16, st, st, &s, 0.1f, fake, fake, fake, nullptr), KSANA_SAGE_EINVAL);
 
   // settings and self-checks
   EXPECT(ksana_sage_configure("kx", KSANA_SAGE_KEEP), KSANA_SAGE_EINVAL);

@@ -357,7 +357,7 @@ int ksana_sage_quant_q(const void* q, int dtype, const int64_t st[4], const ksan
 // row), the row statistic of k is taken along and *k_rms_done says so
 static int quant_q_impl(const void* q, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                         const ksana_sage_prep* prep, float sm_scale, void* ws, void* stream, const void* k,
-                        const int64_t k_st[4], bool* k_rms_done) {
+                        const int64_t k_st[4], bool* k_rms_done, uint16_t* pooled = nullptr) {
   const StageRange range("ksana_sage.quant_q");
   if (k_rms_done) *k_rms_done = false;
   if (int rc = check_shape(s)) return rc;
@@ -387,7 +387,7 @@ static int quant_q_impl(const void* q, int dtype, const int64_t st[4], const ksa
   }
   hipError_t e = ksana_sage::launch_quant_q(in_tensor(q, dtype, st, s->D), s->B, s->Hq, s->Lq, l.lq_pad, premul,
                                             ws_at<int8_t>(ws, l.q_i8), ws_at<float>(ws, l.q_scale),
-                                            static_cast<hipStream_t>(stream), ppp);
+                                            static_cast<hipStream_t>(stream), ppp, pooled);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_q launch");
 }
 
@@ -405,7 +405,7 @@ int ksana_sage_quant_k(const void* k, int dtype, const int64_t st[4], const ksan
 // `rms_done`: the row statistic of k (k_rms area) has been taken by the call before (quant_q_impl)
 static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s,
                         const ksana_sage_prep* prep, int smooth_k, void* ws, float* part, int* sync_words,
-                        void* stream, bool rms_done = false, bool may_allocate = true) {
+                        void* stream, bool rms_done = false, bool may_allocate = true, uint16_t* pooled = nullptr) {
   const StageRange range("ksana_sage.quant_k");
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_tensor("k", k, dtype, st, s->B, s->Lk, s->Hkv)) return rc;
@@ -427,7 +427,7 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
     e = ksana_sage::launch_row_inv_rms(kt, s->B, s->Hkv, s->Lk, prep->norm_eps, ws_at<float>(ws, l.k_rms), hs);
     if (e != hipSuccess) return hip_fail(e, "k row statistic launch");
   }
-  if (one_read('k') || ppp != nullptr) {
+  if ((one_read('k') || ppp != nullptr) && pooled == nullptr) {  // (block averages ride in the two-pass kernel)
     // one read of K: chunk sums, the head's mean and the quantization in one kernel, when the shape suits it (always
     // tried when the step before attention is applied on the way in: the rotation is then done once, not twice)
     e = ksana_sage::launch_clear_ints(sync_words, ksana_sage::sync_words(bhk), hs);
@@ -448,7 +448,7 @@ static int quant_k_impl(const void* k, int dtype, const int64_t st[4], const ksa
                                          ws_at<float>(ws, l.k_mean), hs, sync_at(sync_words, nullptr, bhk).k_status);
   if (e != hipSuccess) return hip_fail(e, "k mean finalize launch");
   e = ksana_sage::launch_quant_k(kt, s->B, s->Hkv, s->Lk, l.nkb, ws_at<float>(ws, l.k_mean),
-                                 ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs, ppp);
+                                 ws_at<int8_t>(ws, l.k_i8), ws_at<float>(ws, l.k_scale), hs, ppp, pooled);
   return e == hipSuccess ? 0 : hip_fail(e, "quant_k launch");
 }
 
@@ -473,6 +473,24 @@ int ksana_sage_quant_qk_prep(const void* q, const void* k, int dtype, const int6
   bool k_rms_done = false;
   if (int rc = quant_q_impl(q, dtype, q_st, s, prep, sm_scale, ws, stream, k, k_st, &k_rms_done)) return rc;
   return quant_k_impl(k, dtype, k_st, s, prep, smooth_k, ws, nullptr, nullptr, stream, k_rms_done);
+}
+
+int ksana_sage_quant_qk_pooled(const void* q, const void* k, int dtype, const int64_t q_st[4], const int64_t k_st[4],
+                               const ksana_sage_shape* s, float sm_scale, void* pooled_q, void* pooled_k, void* ws,
+                               void* stream) {
+  if (int rc = check_shape(s)) return rc;
+  if (s->D != ksana_sage::kD)
+    return fail(KSANA_SAGE_ENOTSUP, "head size %d: the block averages are taken at head size %d only", s->D, ksana_sage::kD);
+  if (pooled_q == nullptr || pooled_k == nullptr) return fail(KSANA_SAGE_EINVAL, "pooled_q / pooled_k is NULL");
+  if ((reinterpret_cast<uintptr_t>(pooled_q) | reinterpret_cast<uintptr_t>(pooled_k)) & 1)
+    return fail(KSANA_SAGE_EINVAL, "pooled_q / pooled_k is not 2-byte aligned");
+  // k is checked before q's kernel goes out: nothing is launched for a call that fails
+  if (int rc = check_tensor("k", k, dtype, k_st, s->B, s->Lk, s->Hkv)) return rc;
+  if (int rc = quant_q_impl(q, dtype, q_st, s, nullptr, sm_scale, ws, stream, nullptr, nullptr, nullptr,
+                            static_cast<uint16_t*>(pooled_q)))
+    return rc;
+  return quant_k_impl(k, dtype, k_st, s, nullptr, 1, ws, nullptr, nullptr, stream, false, true,
+                      static_cast<uint16_t*>(pooled_k));
 }
 
 int ksana_sage_quant_k_static(const void* k, int dtype, const int64_t st[4], const ksana_sage_shape* s, int smooth_k,

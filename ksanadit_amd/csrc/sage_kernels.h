@@ -72,8 +72,11 @@ hipError_t launch_k_mean_finalize(const float* part, int BH, int nch, int L, int
 // zero_mean: nullptr, or the [BH, D] mean slot to clear (V quantized without smoothing)
 hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_scale, float* v_inv, float* zero_mean,
                                    hipStream_t s, int* status = nullptr);
+// pooled (quant_q and quant_k): nullptr, or where the averages of the blocks the kernel quantizes anyway - 128 query
+// rows, 64 keys less their channel mean - go as [B, H, blocks, 128] of the input's half type, bit for bit what
+// launch_block_means gives (head size 128, no prep)
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
-                          float* q_scale, hipStream_t s, const PrepParams* prep = nullptr);
+                          float* q_scale, hipStream_t s, const PrepParams* prep = nullptr, uint16_t* pooled = nullptr);
 // Q with a token-row norm (prep.inv_rms, prep.weight set; kinds 1 and 3): statistic and quantization from one pass over
 // HBM, 32 whole token rows per workgroup; writes prep.inv_rms as launch_row_inv_rms would.  k_rows != nullptr: the
 // statistic of rows [0, k_L) of that tensor (k_H heads of 128 channels, contiguous per row) goes to k_rms on the way.
@@ -81,7 +84,7 @@ hipError_t launch_quant_q_rows(const InTensor& q, int B, int H, int L, int lq_pa
                                int8_t* q_i8, float* q_scale, hipStream_t s, const PrepParams& prep,
                                const InTensor* k_rows, int k_H, int k_L, float* k_rms);
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
-                          float* k_scale, hipStream_t s, const PrepParams* prep = nullptr);
+                          float* k_scale, hipStream_t s, const PrepParams* prep = nullptr, uint16_t* pooled = nullptr);
 // v_mean: nullptr, or the channel means taken off before scaling (V smoothing)
 hipError_t launch_quant_v(const InTensor& v, int B, int H, int L, int nkb, const float* v_inv, const float* v_mean,
                           uint8_t* v_tiles, hipStream_t s);

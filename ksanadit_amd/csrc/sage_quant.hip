@@ -662,16 +662,51 @@ __device__ __forceinline__ uint4 pack_int8x16(const float* x, float inv) {
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// Block mean from per-thread partial sums (thread = row slot x 16 channels; a slot has added its rows in increasing
+// order): the 32 slots meet in an adjacent-pair tree - three steps inside a wave, the four waves through LDS - the sum
+// is divided by the number of rows that exist and rounded to the half type.  The frozen order of the block averages
+// (block_mean_kernel); the quantizers that take a block's average along use the same code, hence give the same bits.
+template <int DT>
+__device__ __forceinline__ void store_block_mean(float (&acc)[16], int t, float n_rows, uint16_t* __restrict__ out_row,
+                                                 float (*s_w)[kD]) {
+  const int c16 = t & 7;
+#pragma unroll
+  for (int m = 8; m <= 32; m <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = acc[e] + __shfl_xor(acc[e], m);
+  }
+  const int wave = t >> 6, lane = t & 63;
+  if (lane < 8) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
+  }
+  __syncthreads();
+  if (t < kD) {
+    const float sum = (s_w[0][t] + s_w[1][t]) + (s_w[2][t] + s_w[3][t]);
+    const float mean = __fdiv_rn(sum, n_rows);
+    uint16_t bits;
+    if constexpr (DT == KSANA_SAGE_BF16) {
+      bits = __builtin_bit_cast(uint16_t, (__bf16)mean);
+    } else {
+      bits = __builtin_bit_cast(uint16_t, (_Float16)mean);
+    }
+    out_row[t] = bits;
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // Q: Hadamard transform, fold sm_scale*log2(e)/128, one int8 scale per query row.  One
 // workgroup handles 128 rows (4 per row slot).  grid = (lq_pad/128, H, B).  Output row-major
 // int8 [B, H, lq_pad, 128] and fp32 [B, H, lq_pad]; rows at or beyond L come out as zeros.
 // ---------------------------------------------------------------------------------------
-template <int DT, int PRE>
+// POOL: the workgroup's 128 rows are one block of the sparse-linear backend's block map; their average (of the input
+// as it is) goes to pooled[b, h, blk, :] - what block_mean_kernel would read q a second time for.
+template <int DT, int PRE, bool POOL = false>
 __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __restrict__ q, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L_all, int d_in, int lq_pad, float premul,
                                                            int8_t* __restrict__ q_i8, float* __restrict__ q_scale,
-                                                           const PrepParams pp) {
+                                                           const PrepParams pp, uint16_t* __restrict__ pooled = nullptr) {
+  static_assert(!(POOL && PRE), "block averages are taken of the tensor as it is");
   const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x, slot = t >> 3, c16 = t & 7;
   const int L = c16 * 16 < d_in ? L_all : 0;  // channels at or past d_in (head size 64) read as zero padding
@@ -719,6 +754,15 @@ __global__ __launch_bounds__(kThreads) void quant_q_kernel(const uint16_t* __res
     for (int i = 0; i < R; ++i) {
       const int row = blk * kRowsPerWg + i * kSlots + slot;
       load_row16<DT>(base + (int64_t)row * sL, row < L, x[i]);
+    }
+    if constexpr (POOL) {
+      float acc[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[e] = ((x[0][e] + x[1][e]) + x[2][e]) + x[3][e];
+      static_assert(R == 4, "four rows per slot");
+      __shared__ float s_w[4][kD];
+      store_block_mean<DT>(acc, t, (float)min(kRowsPerWg, L_all - blk * kRowsPerWg),
+                           pooled + (bh * gridDim.x + blk) * kD, s_w);
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) finish_row(x[i], blk * kRowsPerWg + i * kSlots + slot);
@@ -873,12 +917,16 @@ __global__ __launch_bounds__(kThreads) void quant_q_rows_kernel(const uint16_t* 
 // the attention kernel's int8 MFMA consumes it: fragment (t = row/32, s = 32-channel step)
 // is 64 lanes x 16 bytes, lane = 32*(16-channel half within the step) + row%32.
 // ---------------------------------------------------------------------------------------
-template <int DT, int PRE>
+// POOL: the workgroup's 64 rows are one key block of the sparse-linear backend's block map; the average of
+// k - mean(k), each difference rounded to the tensor's half type first as the reference forms it, goes to
+// pooled[b, h, blk, :] - what block_mean_kernel would read k a third time for.
+template <int DT, int PRE, bool POOL = false>
 __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __restrict__ k, int64_t sB, int64_t sL,
                                                            int64_t sH, int H, int L_all, int d_in, int nkb,
                                                            const float* __restrict__ k_mean,
                                                            int8_t* __restrict__ k_tiles, float* __restrict__ k_scale,
-                                                           const PrepParams pp) {
+                                                           const PrepParams pp, uint16_t* __restrict__ pooled = nullptr) {
+  static_assert(!(POOL && PRE), "block averages are taken of the tensor as it is");
   // Heads and batch entries from the last one down: this pass follows the column-sum pass over the same tensor, which
   // went upwards, so what that pass touched last - and the last-level cache may still hold - is read first.
   const int blk = blockIdx.x, h = (int)gridDim.y - 1 - (int)blockIdx.y, b = (int)gridDim.z - 1 - (int)blockIdx.z;
@@ -893,6 +941,7 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
   const RopeLds rl = maybe_stage_rope<PRE>(pp, b, blk * kBlkK, kBlkK);
   float x[R][16];
   float amax = 0.0f;
+  [[maybe_unused]] float pool_acc[16];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = blk * kBlkK + i * kSlots + slot;
@@ -905,9 +954,20 @@ __global__ __launch_bounds__(kThreads) void quant_k_kernel(const uint16_t* __res
     for (int e = 0; e < 16; ++e) {
       x[i][e] = valid ? x[i][e] - km[e] : 0.0f;
     }
+    if constexpr (POOL) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float d = valid ? through_half<DT>(x[i][e]) : 0.0f;
+        pool_acc[e] = i == 0 ? d : pool_acc[e] + d;
+      }
+    }
     fwht128(x[i], c16);
 #pragma unroll
     for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(x[i][e]));
+  }
+  if constexpr (POOL) {
+    __shared__ float s_w[4][kD];
+    store_block_mean<DT>(pool_acc, t, (float)min(kBlkK, L_all - blk * kBlkK), pooled + (bh * nkb + blk) * kD, s_w);
   }
   __shared__ float s_red[4];
   amax = block_max(amax, s_red);
@@ -1524,31 +1584,8 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(const uint16_t* __
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = i == 0 ? v[e] : acc[e] + v[e];
   }
-#pragma unroll
-  for (int m = 8; m <= 32; m <<= 1) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = acc[e] + __shfl_xor(acc[e], m);
-  }
   __shared__ float s_w[4][kD];
-  const int wave = t >> 6, lane = t & 63;
-  if (lane < 8) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) s_w[wave][c16 * 16 + e] = acc[e];
-  }
-  __syncthreads();
-  if (t < kD) {
-    const float sum = (s_w[0][t] + s_w[1][t]) + (s_w[2][t] + s_w[3][t]);
-    const float n = (float)min(rows, L - blk * rows);
-    const float mean = __fdiv_rn(sum, n);
-    const int64_t nblk = gridDim.x;
-    uint16_t bits;
-    if constexpr (DT == KSANA_SAGE_BF16) {
-      bits = __builtin_bit_cast(uint16_t, (__bf16)mean);
-    } else {
-      bits = __builtin_bit_cast(uint16_t, (_Float16)mean);
-    }
-    out[(bh * nblk + blk) * kD + t] = bits;
-  }
+  store_block_mean<DT>(acc, t, (float)min(rows, L - blk * rows), out + (bh * gridDim.x + blk) * kD, s_w);
 }
 
 __global__ void clear_ints_kernel(int* p, int n) {
@@ -1643,11 +1680,15 @@ hipError_t launch_v_scale_finalize(const float* part, int BH, int nch, float* v_
 }
 
 hipError_t launch_quant_q(const InTensor& q, int B, int H, int L, int lq_pad, float premul, int8_t* q_i8,
-                          float* q_scale, hipStream_t s, const PrepParams* prep) {
+                          float* q_scale, hipStream_t s, const PrepParams* prep, uint16_t* pooled) {
   const dim3 grid(lq_pad / 128, H, B), block(kThreads);
   const PrepParams none{};
+  if (pooled != nullptr && (prep != nullptr || q.D != kD)) return hipErrorInvalidValue;
   KSANA_DISPATCH_DT(q.dtype, {
-    if (prep == nullptr)
+    if (pooled != nullptr)
+      quant_q_kernel<DT, 0, true><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, q.D, lq_pad, premul, q_i8,
+                                                              q_scale, none, pooled);
+    else if (prep == nullptr)
       quant_q_kernel<DT, 0><<<grid, block, 0, s>>>(q.ptr, q.sB, q.sL, q.sH, H, L, q.D, lq_pad, premul, q_i8, q_scale,
                                                         none);
     else {
@@ -1681,11 +1722,15 @@ hipError_t launch_quant_q_rows(const InTensor& q, int B, int H, int L, int lq_pa
 }
 
 hipError_t launch_quant_k(const InTensor& k, int B, int H, int L, int nkb, const float* k_mean, int8_t* k_tiles,
-                          float* k_scale, hipStream_t s, const PrepParams* prep) {
+                          float* k_scale, hipStream_t s, const PrepParams* prep, uint16_t* pooled) {
   const dim3 grid(nkb, H, B), block(kThreads);
   const PrepParams none{};
+  if (pooled != nullptr && (prep != nullptr || k.D != kD)) return hipErrorInvalidValue;
   KSANA_DISPATCH_DT(k.dtype, {
-    if (prep == nullptr)
+    if (pooled != nullptr)
+      quant_k_kernel<DT, 0, true><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb, k_mean, k_tiles,
+                                                              k_scale, none, pooled);
+    else if (prep == nullptr)
       quant_k_kernel<DT, 0><<<grid, block, 0, s>>>(k.ptr, k.sB, k.sL, k.sH, H, L, k.D, nkb, k_mean, k_tiles, k_scale,
                                                         none);
     else {

@@ -412,6 +412,26 @@ def block_means(x: torch.Tensor, rows: int, centre: torch.Tensor | None = None) 
     return out
 
 
+def quant_qk_pooled(q: torch.Tensor, k: torch.Tensor, ws: SageWorkspace, sm_scale: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """``quant_q`` + ``quant_k`` (with K smoothing) that hand back the block averages the sparse-linear backend builds
+    its block map from: ``block_means(q, 128)`` and ``block_means(k, 64, centre=ws.k_mean)``, bit for bit, without the
+    two extra passes over q and k (the quantizers' workgroups are those blocks).  ``[B, L, H, 128]`` tensors."""
+    _require_hip(q, k)
+    if q.dim() != 4 or k.dim() != 4 or q.shape[3] != 128 or k.shape[3] != 128 or q.dtype != k.dtype:
+        raise ValueError("quant_qk_pooled expects [B, L, H, 128] tensors of one dtype")
+    ws.require(q.device, B=q.shape[0], Lq=q.shape[1], Hq=q.shape[2], D=q.shape[3])
+    ws.require(k.device, B=k.shape[0], Lk=k.shape[1], Hkv=k.shape[2], D=k.shape[3])
+    q, k = _usable(q), _usable(k)
+    B, Lq, Hq, D = q.shape
+    pooled_q = torch.empty((B, Hq, -(-Lq // MASK_BLKQ), D), dtype=q.dtype, device=q.device)
+    pooled_k = torch.empty((B, k.shape[2], -(-k.shape[1] // MASK_BLKK), D), dtype=k.dtype, device=k.device)
+    rc = _capi.load().ksana_sage_quant_qk_pooled(q.data_ptr(), k.data_ptr(), _DTYPES[q.dtype], _strides(q), _strides(k),
+                                                 C.byref(ws.shape), sm_scale, pooled_q.data_ptr(), pooled_k.data_ptr(),
+                                                 ws.ptr, _stream_ptr(q.device))
+    _capi.check(rc, "ksana_sage_quant_qk_pooled")
+    return pooled_q, pooled_k
+
+
 def sla_block_map(pooled_q: torch.Tensor, pooled_k: torch.Tensor, keep: int) -> torch.Tensor:
     """int8 ``[B, H, nq, nk]``: per query block ones at the ``keep`` key blocks with the largest
     ``pooled_q @ pooled_k^T`` (a tensor of the blocks' dtype); the second half of ``get_block_map`` (sage_sla.py:83-90).

@@ -396,6 +396,34 @@ def test_block_means_kernel_bit_exact(hip_device, B, L, H, rows, dtype):
         sage_ops.block_means(xd, 48)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Lq,Lk,Hq,Hkv", [(1, 256, 256, 2, 2), (2, 700, 1000, 4, 2), (1, 130, 65, 1, 1)])
+def test_quantizers_take_the_block_averages_along(hip_device, B, Lq, Lk, Hq, Hkv, dtype):
+    """``ksana_sage_quant_qk_pooled``: the quantized operands are bit for bit those of ``quant_q`` + ``quant_k``, and the
+    block averages bit for bit those of the stand-alone kernel (which the test above pins to the oracle) and of the
+    oracle itself - q over 128 rows, ``k - mean(k)`` over 64 (sage_sla.py:43-81, 202-204)."""
+    from oracle.sla_ref import block_means_ref
+
+    print(f"case pooled quantizers B={B} Lq={Lq} Lk={Lk} Hq={Hq} Hkv={Hkv} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(Lq + 7 * Lk)
+    q = (torch.randn((B, Lq, Hq, 128), generator=g) * 1.5).to(dtype)
+    k = (torch.randn((B, Lk, Hkv, 128), generator=g) + torch.randn((1, 1, Hkv, 128), generator=g) * 2.0).to(dtype)
+    qd, kd = q.to(hip_device), k.to(hip_device)
+    sm = 128 ** -0.5
+    ws_a, ws_b = sage_ops.workspace_for(qd, kd), sage_ops.workspace_for(qd, kd)
+    sage_ops.quant_q(qd, ws_a, sm)
+    sage_ops.quant_k(kd, ws_a, True)
+    pq, pk = sage_ops.quant_qk_pooled(qd, kd, ws_b, sm)
+    for name in ("q_i8", "q_scale", "k_tiles", "k_scale", "k_mean"):
+        assert torch.equal(getattr(ws_a, name), getattr(ws_b, name)), name
+    assert torch.equal(pq, sage_ops.block_means(qd, 128))
+    assert torch.equal(pk, sage_ops.block_means(kd, 64, centre=ws_a.k_mean))
+    assert torch.equal(pq.cpu(), block_means_ref(q.permute(0, 2, 1, 3), 128))
+    assert torch.equal(pk.cpu(), block_means_ref(k.permute(0, 2, 1, 3), 64, centre=ws_a.k_mean.cpu()))
+    with pytest.raises(ValueError):
+        sage_ops.quant_qk_pooled(qd[..., :64], kd[..., :64], ws_b, sm)
+
+
 def test_sla_backend_sparse_plus_linear(hip_device):
     """sage_sla.py:141-292: dense when asked, else block-sparse attention on the top-k map plus the projected
     linear branch.  The map, the linear branch and the composition are checked against the oracle's own restatements
