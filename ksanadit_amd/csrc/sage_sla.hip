@@ -508,10 +508,12 @@ __global__ __launch_bounds__(kSlaThreads) void sla_block_map_kernel(const uint16
 
 }  // namespace
 
-// rows per run of sla_kv_partial_kernel: about two workgroups per compute unit in all, runs a multiple of 128 rows
+// rows per run of sla_kv_partial_kernel, runs a multiple of 128 rows: as many runs per head as keep the whole grid
+// within the 512 workgroups the chip holds at once (two per compute unit, 64 KiB of LDS each) - a few workgroups
+// more than that and the launch takes two rounds for one round's work (520 workgroups: 212 us; 480: see profiles)
 void plan_sla_runs(int B, int H, int L, int* runs, int* rows_per_run) {
   const int steps = (L + kSlaStepRows - 1) / kSlaStepRows;
-  int n = (512 + B * H - 1) / (B * H);
+  int n = 512 / max(1, B * H);
   n = max(1, min(n, steps));
   const int steps_per_run = (steps + n - 1) / n;
   *rows_per_run = steps_per_run * kSlaStepRows;
