@@ -473,6 +473,55 @@ def test_sla_backend_sparse_plus_linear(hip_device):
     assert (out.float() - ref).abs().max() <= 0.1 * max(ref.abs().max().item(), 0.1)
 
 
+def test_sla_backend_at_the_headline_shape(hip_device):
+    """The sparse-linear backend (sage_sla.py:141-292) at wan14b_480p's length, two heads of its seeded inputs, topk
+    0.10, against the CPU oracle: the block averages at full size bit for bit; the map as a valid top-k of the oracle's
+    scores (equal scores at the cut may fall either way); the output on sampled query blocks against masked SDPA on
+    the map the device built plus the projected linear branch."""
+    from ksanadit_amd.config import KsanaSageSLAConfig
+    from oracle.quant_ref import k_mean_ref
+    from oracle.sla_ref import block_means_ref, linear_branch_ref
+
+    q, k, v = make_inputs("wan14b_480p", heads=2)
+    B, L, H, D = q.shape
+    print(f"case sla headline B={B} L={L} H={H}", flush=True)
+    qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
+    topk = 0.1
+    op = pick_attn_op(KsanaSageSLAConfig(topk=topk))(num_heads=H, head_size=D, causal=False)
+    proj = torch.nn.Linear(D, D, bias=True).to(hip_device).to(q.dtype)
+    torch.nn.init.normal_(proj.weight, std=0.05)
+    with torch.no_grad():
+        out = op(qd, kd, vd, proj_l=proj).cpu()
+    assert out.shape == q.shape and torch.isfinite(out.float()).all()
+    # block averages and map, as the backend builds them
+    ws = sage_ops.workspace_for(qd, kd)
+    pq, pk = sage_ops.quant_qk_pooled(qd, kd, ws, D ** -0.5)
+    qh, kh = q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3)
+    want_pq, want_pk = block_means_ref(qh, 128), block_means_ref(kh, 64, centre=k_mean_ref(k))
+    assert torch.equal(pq.cpu(), want_pq) and torch.equal(pk.cpu(), want_pk)
+    nk = pk.shape[2]
+    keep = int(topk * nk)
+    bm = sage_ops.sla_block_map(pq, pk, keep).cpu()
+    assert bm.shape == (B, H, pq.shape[2], nk) and bool((bm.sum(-1) == keep).all())
+    score = (want_pq.float() @ want_pk.float().transpose(-1, -2)).to(q.dtype).float()
+    lowest_kept = torch.where(bm != 0, score, torch.full_like(score, float("inf"))).amin(-1)
+    highest_dropped = torch.where(bm == 0, score, torch.full_like(score, float("-inf"))).amax(-1)
+    assert bool((lowest_kept >= highest_dropped).all()), "a dropped key block outscores a kept one"
+    # the output on eight query blocks spread over the sequence
+    blocks = [0, 1, 37, 100, 128, 200, 254, pq.shape[2] - 1]
+    with torch.no_grad():
+        lin = proj.cpu().float()(linear_branch_ref(q, k, v).float()).transpose(1, 2)  # [B, L, H, D]
+    worst, cos_min = 0.0, 1.0
+    for i in blocks:
+        rows = slice(128 * i, min(L, 128 * (i + 1)))
+        ref = sdpa_ref(q[:, rows], k, v, block_mask=bm[:, :, i:i + 1]).float() + lin[:, rows]
+        got = out[:, rows].float()
+        cos_min = min(cos_min, _cos(got, ref))
+        worst = max(worst, ((got - ref).abs().max() / ref.abs().max()).item())
+    print(f"sla headline: cos >= {cos_min:.6f}, worst element {worst:.4f} of the block's max", flush=True)
+    assert cos_min >= COS_MIN and worst <= 0.2
+
+
 @pytest.mark.parametrize("B,H,nq,nk,keep,dtype", [(1, 2, 45, 70, 9, torch.bfloat16), (2, 3, 8, 512, 51, torch.float16),
                                                    (1, 1, 33, 1024, 1, torch.bfloat16), (1, 2, 16, 96, 0, torch.bfloat16),
                                                    (1, 2, 16, 96, 96, torch.bfloat16), (1, 40, 256, 512, 51, torch.bfloat16)])
