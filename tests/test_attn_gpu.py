@@ -1017,22 +1017,29 @@ def test_randomized_shapes_and_options(hip_device):
     import random
 
     rng = random.Random(20240607)
-    for case in range(28):
-        B = rng.choice([1, 1, 2, 3])
-        Hkv = rng.choice([1, 2, 3])
+    for case in range(40):
+        # the last twelve: key sequences of 16 - 47 tiles, mostly with a tile list (block mask or causal), so that the
+        # list walk is long enough for its look-ahead to wrap, with query blocks whose last waves have no rows
+        long_keys = case >= 28
+        B = rng.choice([1, 1, 2, 3]) if not long_keys else rng.choice([1, 2])
+        Hkv = rng.choice([1, 2, 3]) if not long_keys else rng.choice([1, 2])
         Hq = Hkv * rng.choice([1, 1, 2])
         causal = rng.random() < 0.3
-        Lk = rng.choice([1, 7, 63, 64, 65, 127, 130, 255, 256, 300, 511, 640, 777])
-        Lq = Lk if causal else rng.choice([1, 31, 32, 33, 100, 255, 256, 257, 290, 513])
+        if long_keys:
+            Lk = rng.choice([1000, 1500, 2047, 2100, 3000])
+            Lq = Lk if causal else rng.choice([100, 257, 300, 700])
+        else:
+            Lk = rng.choice([1, 7, 63, 64, 65, 127, 130, 255, 256, 300, 511, 640, 777])
+            Lq = Lk if causal else rng.choice([1, 31, 32, 33, 100, 255, 256, 257, 290, 513])
         dtype = rng.choice([torch.bfloat16, torch.float16])
         exact = rng.random() < 0.6
         k_lens = [rng.randint(0, Lk + 3) for _ in range(B)] if rng.random() < 0.4 else None
         mask = None
-        if rng.random() < 0.4:
+        if rng.random() < (0.8 if long_keys else 0.4):
             nq, nk = -(-Lq // 128), -(-Lk // 64)
             g = torch.Generator().manual_seed(case)
             lead = rng.choice([(), (Hq,), (B, Hq), (B, 1)])
-            mask = (torch.rand((*lead, nq, nk), generator=g) < 0.6).to(torch.int8)
+            mask = (torch.rand((*lead, nq, nk), generator=g) < (rng.choice([0.15, 0.4, 0.9]) if long_keys else 0.6)).to(torch.int8)
         print(f"case {case}: B={B} Hq={Hq} Hkv={Hkv} Lq={Lq} Lk={Lk} {dtype} exact={exact} causal={causal} k_lens={k_lens} "
               f"mask={None if mask is None else tuple(mask.shape)}", flush=True)
         q, k, v = _rand_qkv(B, Lq, Lk, Hq, Hkv, seed=1000 + case, dtype=dtype)
