@@ -78,7 +78,7 @@ constexpr float kMagicF2 = 25165824.0f;
 constexpr float kPShift = 6.0f, kPShiftPwl = 8.0f;
 constexpr float kLazyMax = 2.7f, kLazyMaxPwl = 0.0f;
 constexpr int kStageBytes = 2 * kTileBytes;  // K tile + V tile
-constexpr int kSparseMaxKeyTiles4 = 1024;    // 4-wave workgroups keep a shorter tile list so that two fit a compute unit
+constexpr int kSparseMaxKeyTiles4 = 2048;    // 4-wave workgroups keep their tile list as 16-bit entries so that two fit a compute unit
 constexpr int kMaxKeyTiles = 4096;           // K scales of one head are kept in LDS: Lk <= 262144
 constexpr int kShortKeyTiles = 16;           // dense calls with at most this many key tiles (Lk <= 1024) take 4-wave workgroups
 constexpr int kShortMaxKeyTiles = 2048;      // the most key tiles a dense 4-wave workgroup can hold scales for
@@ -303,7 +303,11 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
   // Causal attention (key <= query row) runs through the same list: the workgroup lists the tiles up
   // to the one holding its last row, a wave leaves alone the tiles past its own last row, and the one
   // tile that straddles its rows' diagonal is masked element by element.
-  int* s_list = reinterpret_cast<int*>(s_ks + kListMax);
+  // (one mask row per 4-wave workgroup: an entry is the tile number and fits 16 bits; with two mask rows per
+  // workgroup it carries their two flags above the number)
+  using ListEntry = typename std::conditional<kW == 4, uint16_t, int>::type;
+  ListEntry* s_list = reinterpret_cast<ListEntry*>(s_ks + kListMax);
+  int* s_count = reinterpret_cast<int*>(s_list + kListMax);
   int n_tiles = nkb;  // loop length: list entries with a mask, key tiles without
   // a wave's 32 rows start at a multiple of 32, so exactly one 64-key tile holds their diagonal
   const int my_last = (kSparse && causal) ? (q0 >> 6) : 0x7fffffff;
@@ -341,14 +345,14 @@ __global__ __launch_bounds__(kW * 64, kW == 8 ? 1 : 2) void sage_attn_fwd_kernel
           const bool keep = (f0 | f1) != 0;
           const unsigned long long bal = __ballot(keep);
           const int pre = __builtin_amdgcn_mbcnt_hi((unsigned)(bal >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)bal, 0));
-          if (keep) s_list[base + pre] = j | (f0 << 16) | (f1 << 17);
+          if (keep) s_list[base + pre] = static_cast<ListEntry>(kW == 4 ? j : (j | (f0 << 16) | (f1 << 17)));
           base += __popcll(bal);
         }
       }
-      if (lane == 0) s_list[kListMax] = base;
+      if (lane == 0) *s_count = base;
     }
     __syncthreads();
-    n_tiles = __builtin_amdgcn_readfirstlane(s_list[kListMax]);
+    n_tiles = __builtin_amdgcn_readfirstlane(*s_count);
     if (n_tiles == 0) {  // neither mask row allows any key
       write_zero_rows();
       return;
@@ -906,7 +910,7 @@ __global__ __launch_bounds__(256) void sage_attn_merge_kernel(const AttnParams p
 // dynamic LDS of one instantiation: tile ring + K scales (+ the tile list and its length with a mask or causal)
 template <bool kSparse, int kW>
 constexpr size_t max_lds() {
-  return kSparse ? WgShape<kW>::kRingBytes + 1024 + 2 * (kW == 8 ? kSparseMaxKeyTiles : kSparseMaxKeyTiles4) * 4 + 1024
+  return kSparse ? WgShape<kW>::kRingBytes + 1024 + (kW == 8 ? kSparseMaxKeyTiles * 8 : kSparseMaxKeyTiles4 * 6) + 1024
                  : WgShape<kW>::kRingBytes + 1024 + (kW == 8 ? kMaxKeyTiles : kShortMaxKeyTiles) * 4;
 }
 
@@ -1014,7 +1018,7 @@ hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
   const int n_wg = p.B * p.Hq * n_qwg;
   const int wg_per_xcd = (n_wg + 7) / 8;
   const dim3 grid(wg_per_xcd * 8);
-  // (beyond 65 536 keys with a mask: one instantiation serves causal and plain calls)
+  // (tile lists in 256-row workgroups, by flag only: one instantiation serves causal and plain calls)
   if (sparse) return launch_shape<true, false, 8, true>(p, grid, max_lds<true, 8>(), n_qwg, n_wg, wg_per_xcd, s);
   // tile ring + the head's K scales (a multiple of 1 KiB keeps the request tidy)
   const size_t lds = WgShape<8>::kRingBytes + 1024 + (((size_t)p.nkb * 4 + 1023) & ~size_t(1023));

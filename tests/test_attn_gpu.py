@@ -488,8 +488,12 @@ def test_sla_backend_at_the_headline_shape(hip_device):
     qd, kd, vd = (t.to(hip_device) for t in (q, k, v))
     topk = 0.1
     op = pick_attn_op(KsanaSageSLAConfig(topk=topk))(num_heads=H, head_size=D, causal=False)
-    proj = torch.nn.Linear(D, D, bias=True).to(hip_device).to(q.dtype)
-    torch.nn.init.normal_(proj.weight, std=0.05)
+    proj = torch.nn.Linear(D, D, bias=True)
+    g = torch.Generator().manual_seed(83)
+    with torch.no_grad():
+        proj.weight.copy_(0.05 * torch.randn((D, D), generator=g))
+        proj.bias.copy_(0.05 * torch.randn(D, generator=g))
+    proj = proj.to(hip_device).to(q.dtype)
     with torch.no_grad():
         out = op(qd, kd, vd, proj_l=proj).cpu()
     assert out.shape == q.shape and torch.isfinite(out.float()).all()
