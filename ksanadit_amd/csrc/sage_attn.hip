@@ -81,6 +81,7 @@ constexpr int kStageBytes = 2 * kTileBytes;  // K tile + V tile
 constexpr int kSparseMaxKeyTiles4 = 2048;    // 4-wave workgroups keep their tile list as 16-bit entries so that two fit a compute unit
 constexpr int kMaxKeyTiles = 4096;           // K scales of one head are kept in LDS: Lk <= 262144
 constexpr int kShortKeyTiles = 16;           // dense calls with at most this many key tiles (Lk <= 1024) take 4-wave workgroups
+constexpr int kMidKeyTiles = 96;             // ... and up to this many (Lk <= 6144) when their 256-row grid fills the chip at least once
 constexpr int kShortMaxKeyTiles = 2048;      // the most key tiles a dense 4-wave workgroup can hold scales for
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -969,8 +970,17 @@ int compute_units() {
 
 }  // namespace
 
+// Dense calls that take 4-wave workgroups (n_wg8: their grid in 256-row workgroups): short key loops, where a
+// workgroup's fixed costs weigh as much as its loop and hide under the compute unit's other workgroup - measured at
+// B * H = 40 and 48: 32 tiles 14-19 % faster than 256-row workgroups, 64-68 tiles 2-6 %, 128 tiles 1-3 % slower.
+// Beyond kShortKeyTiles only when the chip is full anyway: a grid of a few workgroups is better off cut into runs of
+// keys, which only the 256-row shape does.
+static bool dense_in_four_waves(int n_wg8, int nkb) {
+  return nkb <= kShortKeyTiles || (nkb <= kMidKeyTiles && n_wg8 >= compute_units());
+}
+
 void plan_key_split(int n_wg, int nkb, int* first_wg, int* runs) {
-  if (nkb <= kShortKeyTiles) {  // these shapes run in 4-wave workgroups, which are never cut
+  if (dense_in_four_waves(n_wg, nkb)) {  // these shapes run in 4-wave workgroups, which are never cut
     *first_wg = n_wg, *runs = 0;
     return;
   }
@@ -987,14 +997,14 @@ void plan_key_split(int n_wg, int nkb, int* first_wg, int* runs) {
 
 // Workgroup shape for a call: 4-wave workgroups (two per compute unit) when a block mask or causal masking is
 // involved (a workgroup is then one 128-row mask row, so no wave multiplies a tile only the neighbouring mask row
-// asked for) and for short key sequences (a workgroup's fixed costs - operand loads, first copies, the output store -
-// then weigh as much as its key loop and hide under the other workgroup's); 8-wave workgroups otherwise, which copy
+// asked for) and for short key sequences (dense_in_four_waves); 8-wave workgroups otherwise, which copy
 // every K/V tile once per 256 rows instead of once per 128.  p.wg_waves (4 or 8) overrides the choice.
 static int pick_wg_waves(const AttnParams& p) {
   if (p.wg_waves == 4 || p.wg_waves == 8) return p.wg_waves;
   const bool sparse = p.block_mask != nullptr || p.causal;
   if (sparse) return p.nkb <= kSparseMaxKeyTiles4 ? 4 : 8;
-  return p.nkb <= kShortKeyTiles ? 4 : 8;
+  const int n_wg8 = p.B * p.Hq * ((p.Lq + kAttnQPerWg - 1) / kAttnQPerWg);
+  return dense_in_four_waves(n_wg8, p.nkb) ? 4 : 8;
 }
 
 hipError_t launch_attn_fwd(const AttnParams& p, hipStream_t s) {
