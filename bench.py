@@ -210,6 +210,16 @@ def other_workloads(sage_ops, dev, pwl, iters=7):
                        "attn_kernel_tflops": round(flops / (ms * 1e-3) / 1e12, 1),
                        "frac_of_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
                        "quantizer_ms": round(ev[0].elapsed_time(ev[1]), 4)}
+        if w.name == "wan14b_720p":
+            # tile lists of more than 1 024 entries (1 182 key tiles): a radial-style mask and causal masking
+            mask = radial_style_mask(w.L, WAN_GRIDS[w.name]).to(dev)
+            density = float(mask.float().mean())
+            t_mask = pctl(time_attention(sage_ops, ws, out, 3, pwl_exp2=pwl, block_mask=mask), 0.5)
+            t_causal = pctl(time_attention(sage_ops, ws, out, 3, pwl_exp2=pwl, causal=True), 0.5)
+            res[w.name]["block_sparse"] = {"density": round(density, 4), "attn_kernel_ms": round(t_mask, 4),
+                                           "kept_block_rate_vs_dense": round(density * ms / t_mask, 3)}
+            res[w.name]["causal"] = {"attn_kernel_ms": round(t_causal, 4),
+                                     "kept_pair_rate_vs_dense": round((w.L + 1) / (2.0 * w.L) * ms / t_causal, 3)}
         del q, k, v, ws, out
         torch.cuda.empty_cache()
     # Head size 64 (no BASELINE model has it; the backend interface serves it): the headline shape's token count
