@@ -994,6 +994,11 @@ def test_maximum_key_lengths(hip_device):
     qd, kd, vd = q.to(hip_device), k.to(hip_device), v.to(hip_device)
     out = sage_ops.sageattn(qd, kd, vd, block_mask=mask).cpu()
     assert _cos(out, sdpa_ref(q.float(), k.float(), v.float(), block_mask=mask)) >= COS_MIN
+    # the same call in 256-row workgroups (two mask rows share a tile list; selected by flag only): same bits
+    ws = sage_ops.workspace_for(qd, kd)
+    sage_ops.quant_q(qd, ws, 128 ** -0.5), sage_ops.quant_k(kd, ws, True), sage_ops.quant_v(vd, ws)
+    by_shape = [sage_ops.attn_fwd(ws, torch.empty_like(qd), block_mask=mask.to(hip_device), wg_waves=w).cpu() for w in (4, 8)]
+    assert torch.equal(by_shape[0], by_shape[1]) and torch.equal(by_shape[0], out)
     with pytest.raises(NotImplementedError):
         sage_ops.sageattn(qd, torch.cat([kd, kd[:, :1]], dim=1), torch.cat([vd, vd[:, :1]], dim=1),
                           block_mask=torch.ones(4, 2049, dtype=torch.int8))
