@@ -398,7 +398,7 @@ def test_block_means_kernel_bit_exact(hip_device, B, L, H, rows, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,Lq,Lk,Hq,Hkv", [(1, 256, 256, 2, 2), (2, 700, 1000, 4, 2), (1, 130, 65, 1, 1)])
-def test_quantizers_take_the_block_averages_along(hip_device, B, Lq, Lk, Hq, Hkv, dtype):
+def test_quantizers_take_the_block_averages_along(hip_device, quant_settings, B, Lq, Lk, Hq, Hkv, dtype):
     """``ksana_sage_quant_qk_pooled``: the quantized operands are bit for bit those of ``quant_q`` + ``quant_k``, and the
     block averages bit for bit those of the stand-alone kernel (which the test above pins to the oracle) and of the
     oracle itself - q over 128 rows, ``k - mean(k)`` over 64 (sage_sla.py:43-81, 202-204)."""
@@ -422,6 +422,14 @@ def test_quantizers_take_the_block_averages_along(hip_device, B, Lq, Lk, Hq, Hkv
     assert torch.equal(pk.cpu(), block_means_ref(k.permute(0, 2, 1, 3), 64, centre=ws_a.k_mean.cpu()))
     with pytest.raises(ValueError):
         sage_ops.quant_qk_pooled(qd[..., :64], kd[..., :64], ws_b, sm)
+    # with the one-read K quantizer switched on for plain calls, this call still takes the two-pass kernels (the
+    # averages ride in their second pass): same results
+    quant_settings(one_read="kv")
+    ws_c = sage_ops.workspace_for(qd, kd)
+    pq2, pk2 = sage_ops.quant_qk_pooled(qd, kd, ws_c, sm)
+    assert torch.equal(pq2, pq) and torch.equal(pk2, pk)
+    for name in ("k_tiles", "k_scale", "k_mean"):
+        assert torch.equal(getattr(ws_c, name), getattr(ws_a, name)), name
 
 
 def test_sla_backend_sparse_plus_linear(hip_device):
